@@ -1,0 +1,244 @@
+// Torch bindings of the dtype-generic kernels (csrc/kernels/mix_ops.hip, latent_attn.hip) and of the expert
+// alignment kernel they share with the Mixtral path (moe.hip). Built as src/_Cmix: a model that needs only
+// these compiles only these. Shapes, dtypes and devices are validated here; the launchers trust them.
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include "kernels/launchers.h"
+#include "kernels/mix_launchers.h"
+
+using at::Tensor;
+using OptTensor = c10::optional<Tensor>;
+
+namespace {
+
+inline hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+#define HIP_OK(call)                                                                                   \
+  do {                                                                                                  \
+    hipError_t e_ = (call);                                                                             \
+    TORCH_CHECK(e_ == hipSuccess, "HIP launch failed: ", hipGetErrorString(e_), " (", #call, ")");      \
+  } while (0)
+
+// storage type of an activation / weight tensor: true = fp32, false = bf16
+bool is_f32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, name, " must be bf16 or fp32");
+  return t.scalar_type() == at::kFloat;
+}
+
+void check_rows(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 2 && t.stride(1) == 1, name, " must be [rows, n] with unit inner stride");
+}
+
+void check_i(const Tensor& t, at::ScalarType d, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == d && t.is_contiguous(), name, ": wrong device / dtype / layout");
+}
+
+void rms_norm_ext(Tensor out, Tensor x, OptTensor w, bool unit_offset, double eps) {
+  check_rows(out, "out");
+  check_rows(x, "x");
+  const bool of = is_f32(out, "out"), xf = is_f32(x, "x");
+  TORCH_CHECK(out.size(0) == x.size(0) && out.size(1) == x.size(1), "rms_norm_ext shapes");
+  bool wf = false;
+  const void* wp = nullptr;
+  if (w.has_value()) {
+    wf = is_f32(*w, "w");
+    TORCH_CHECK(w->is_contiguous() && w->numel() == x.size(1), "w [n]");
+    wp = w->data_ptr();
+  }
+  HIP_OK(die::launch_rms_norm_ext(out.data_ptr(), out.stride(0), of, x.data_ptr(), x.stride(0), xf, wp, wf,
+                                  unit_offset, (float)eps, (int)x.size(0), (int)x.size(1), cur_stream()));
+}
+
+void post_norm_residual(Tensor resid, OptTensor act, Tensor y, Tensor w, bool unit_offset, double eps) {
+  TORCH_CHECK(resid.is_cuda() && resid.scalar_type() == at::kFloat && resid.is_contiguous() && resid.dim() == 2,
+              "resid must be a contiguous fp32 [rows, n] GPU tensor");
+  check_rows(y, "y");
+  const bool yf = is_f32(y, "y"), wf = is_f32(w, "w");
+  TORCH_CHECK(y.size(0) == resid.size(0) && y.size(1) == resid.size(1) && w.is_contiguous() &&
+                  w.numel() == resid.size(1),
+              "post_norm_residual shapes");
+  void* ap = nullptr;
+  if (act.has_value()) {
+    TORCH_CHECK(act->is_cuda() && act->scalar_type() == at::kBFloat16 && act->is_contiguous() &&
+                    act->sizes() == resid.sizes(),
+                "act must be a contiguous bf16 tensor of the residual's shape");
+    ap = act->data_ptr();
+  }
+  HIP_OK(die::launch_post_norm_residual(resid.data_ptr<float>(), ap, y.data_ptr(), y.stride(0), yf, w.data_ptr(), wf,
+                                        unit_offset, (float)eps, (int)resid.size(0), (int)resid.size(1),
+                                        cur_stream()));
+}
+
+void gated_act(Tensor out, Tensor gu, int64_t kind, double limit, double alpha) {
+  const bool f = is_f32(gu, "gu");
+  TORCH_CHECK(is_f32(out, "out") == f && out.is_contiguous() && gu.is_contiguous() && gu.dim() == 2 &&
+                  out.dim() == 2 && gu.size(1) == 2 * out.size(1) && gu.size(0) == out.size(0),
+              "gated_act: gu [rows, 2f] -> out [rows, f], same dtype, contiguous");
+  HIP_OK(die::launch_gated_act(out.data_ptr(), gu.data_ptr(), f, (int)out.size(0), (int)out.size(1), (int)kind,
+                               (float)limit, (float)alpha, cur_stream()));
+}
+
+void route_sigmoid_topk(Tensor w, Tensor ids, Tensor x, Tensor wr) {
+  check_rows(x, "x");
+  const bool xf = is_f32(x, "x"), wf = is_f32(wr, "wr");
+  check_i(w, at::kFloat, "w");
+  check_i(ids, at::kInt, "ids");
+  TORCH_CHECK(wr.dim() == 2 && wr.is_contiguous() && wr.size(1) == x.size(1), "wr [E, H]");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == x.size(0) && ids.sizes() == w.sizes() && w.size(1) <= wr.size(0),
+              "w, ids [T, K], K <= E");
+  HIP_OK(die::launch_route_sigmoid_topk(w.data_ptr<float>(), ids.data_ptr<int>(), x.data_ptr(), x.stride(0), xf,
+                                        wr.data_ptr(), wf, (int)x.size(0), (int)x.size(1), (int)wr.size(0),
+                                        (int)w.size(1), cur_stream()));
+}
+
+void gather_scaled(Tensor xs, Tensor x, OptTensor sorted, Tensor w, int64_t topk) {
+  const bool f = is_f32(x, "x");
+  check_i(w, at::kFloat, "w");
+  TORCH_CHECK(is_f32(xs, "xs") == f && xs.is_contiguous() && x.is_contiguous() && xs.dim() == 2 && x.dim() == 2 &&
+                  xs.size(1) == x.size(1) && xs.size(0) == x.size(0) * topk && w.numel() == xs.size(0),
+              "gather_scaled shapes");
+  const int* sp = nullptr;
+  if (sorted.has_value()) {
+    check_i(*sorted, at::kInt, "sorted");
+    TORCH_CHECK(sorted->numel() == xs.size(0), "sorted [T * K]");
+    sp = sorted->data_ptr<int>();
+  }
+  HIP_OK(die::launch_gather_scaled(xs.data_ptr(), x.data_ptr(), f, sp, w.data_ptr<float>(), (int)xs.size(0),
+                                   (int)topk, (int)x.size(1), cur_stream()));
+}
+
+void combine_sum(Tensor out, Tensor ys, OptTensor pos, OptTensor extra, int64_t topk) {
+  const bool f = is_f32(ys, "ys");
+  check_i(out, at::kFloat, "out");
+  TORCH_CHECK(out.dim() == 2 && ys.dim() == 2 && ys.is_contiguous() && ys.size(1) == out.size(1) &&
+                  ys.size(0) == out.size(0) * topk,
+              "combine_sum shapes");
+  const int* pp = nullptr;
+  if (pos.has_value()) {
+    check_i(*pos, at::kInt, "pos");
+    TORCH_CHECK(pos->numel() == ys.size(0), "pos [T * K]");
+    pp = pos->data_ptr<int>();
+  }
+  const void* ep = nullptr;
+  if (extra.has_value()) {
+    TORCH_CHECK(is_f32(*extra, "extra") == f && extra->is_contiguous() && extra->sizes() == out.sizes(),
+                "extra: same dtype as ys, shape of out");
+    ep = extra->data_ptr();
+  }
+  HIP_OK(die::launch_combine_sum(out.data_ptr<float>(), ys.data_ptr(), f, pp, ep, (int)out.size(0), (int)topk,
+                                 (int)out.size(1), cur_stream()));
+}
+
+die::LatentShape latent_shape(int64_t rank, int64_t rot_dim, const Tensor& inv_freq) {
+  check_i(inv_freq, at::kFloat, "inv_freq");
+  TORCH_CHECK(rank >= 1 && rot_dim >= 0 && inv_freq.numel() * 2 <= rot_dim, "latent shape");
+  die::LatentShape sh;
+  sh.rank = (int)rank;
+  sh.rot_dim = (int)rot_dim;
+  sh.rot_pairs = (int)inv_freq.numel();
+  sh.inv_freq = inv_freq.data_ptr<float>();
+  return sh;
+}
+
+// cache [num_blocks, block_size, rank + rot_dim]; kv [T, >= rank + rot_dim]
+void latent_kv_write(Tensor cache, Tensor kv, Tensor w, Tensor positions, Tensor slots, int64_t rank, int64_t rot_dim,
+                     Tensor inv_freq, double eps) {
+  check_rows(kv, "kv");
+  const bool f = is_f32(kv, "kv"), wf = is_f32(w, "w");
+  TORCH_CHECK(is_f32(cache, "cache") == f && cache.is_contiguous() && cache.dim() == 3 &&
+                  cache.size(2) == rank + rot_dim && kv.size(1) == rank + rot_dim,
+              "latent_kv_write: cache [blocks, block_size, rank + rot_dim], kv [T, rank + rot_dim], same dtype");
+  TORCH_CHECK(w.is_contiguous() && w.numel() == rank, "w [rank]");
+  check_i(positions, at::kLong, "positions");
+  check_i(slots, at::kLong, "slots");
+  TORCH_CHECK(positions.numel() >= kv.size(0) && slots.numel() >= kv.size(0), "positions / slots [T]");
+  HIP_OK(die::launch_latent_kv_write(cache.data_ptr(), kv.data_ptr(), kv.stride(0), f, w.data_ptr(), wf,
+                                     positions.data_ptr<int64_t>(), slots.data_ptr<int64_t>(), (int)kv.size(0),
+                                     latent_shape(rank, rot_dim, inv_freq), (float)eps, cur_stream()));
+}
+
+// out, q_lat [H, T, rank]; q [T, H * qh] whose head h keeps its rotary part at [h * qh + rot_off, + rot_dim)
+void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cache, Tensor block_tables,
+                 OptTensor cu_q, Tensor ctx_lens, Tensor positions, OptTensor sink, int64_t max_q, int64_t window,
+                 double scale, int64_t rot_dim, Tensor inv_freq) {
+  const bool f = is_f32(q_lat, "q_lat");
+  TORCH_CHECK(is_f32(out, "out") == f && is_f32(q, "q") == f && is_f32(cache, "cache") == f, "one dtype");
+  TORCH_CHECK(q_lat.dim() == 3 && q_lat.is_contiguous() && out.is_contiguous() && out.sizes() == q_lat.sizes(),
+              "q_lat, out [H, T, rank] contiguous");
+  const int64_t H = q_lat.size(0), T = q_lat.size(1), rank = q_lat.size(2);
+  check_rows(q, "q");
+  TORCH_CHECK(q.size(0) == T && q.size(1) % H == 0, "q [T, H * qh]");
+  const int64_t qh = q.size(1) / H;
+  TORCH_CHECK(rot_off >= 0 && rot_off + rot_dim <= qh, "rotary part outside the head");
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && cache.size(2) == rank + rot_dim, "cache layout");
+  check_i(ctx_lens, at::kInt, "ctx_lens");
+  check_i(positions, at::kLong, "positions");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
+                  block_tables.stride(1) == 1,
+              "block_tables [S, W] int32");
+  const int64_t S = block_tables.size(0);
+  TORCH_CHECK(ctx_lens.numel() >= S && positions.numel() >= T, "ctx_lens [S], positions [T]");
+  die::LatentAttnArgs a;
+  a.out = out.data_ptr();
+  a.q_lat = q_lat.data_ptr();
+  a.q_rot = static_cast<const char*>(q.data_ptr()) + rot_off * q.element_size();
+  a.q_stride = q.stride(0);
+  a.q_hstride = qh;
+  a.cache = cache.data_ptr();
+  a.block_tables = block_tables.data_ptr<int>();
+  a.bt_stride = (int)block_tables.stride(0);
+  a.cu_q = nullptr;
+  if (cu_q.has_value()) {
+    check_i(*cu_q, at::kInt, "cu_q");
+    TORCH_CHECK(cu_q->numel() >= S + 1, "cu_q [S + 1]");
+    a.cu_q = cu_q->data_ptr<int>();
+  } else {
+    TORCH_CHECK(T >= S && max_q == 1, "without cu_q every sequence has one row");
+  }
+  a.ctx_lens = ctx_lens.data_ptr<int>();
+  a.positions = positions.data_ptr<int64_t>();
+  a.sink = nullptr;
+  if (sink.has_value()) {
+    check_i(*sink, at::kFloat, "sink");
+    TORCH_CHECK(sink->numel() == H, "sink [H]");
+    a.sink = sink->data_ptr<float>();
+  }
+  a.num_seqs = (int)S;
+  a.total_q = (int)T;
+  a.max_q = (int)max_q;
+  a.heads = (int)H;
+  a.block_size = (int)cache.size(1);
+  a.window = (int)window;
+  a.scale = (float)scale;
+  a.sh = latent_shape(rank, rot_dim, inv_freq);
+  a.f32 = f;
+  HIP_OK(die::launch_latent_attn(a, cur_stream()));
+}
+
+void moe_align(Tensor offsets, Tensor sorted, Tensor pos, Tensor ids, int64_t num_experts) {
+  check_i(offsets, at::kInt, "offsets");
+  check_i(sorted, at::kInt, "sorted");
+  check_i(pos, at::kInt, "pos");
+  check_i(ids, at::kInt, "ids");
+  TORCH_CHECK(offsets.numel() >= num_experts + 1 && sorted.numel() >= ids.numel() && pos.numel() >= ids.numel(),
+              "moe_align buffers");
+  HIP_OK(die::launch_moe_align(offsets.data_ptr<int>(), sorted.data_ptr<int>(), pos.data_ptr<int>(),
+                               ids.data_ptr<int>(), (int)ids.numel(), (int)num_experts, cur_stream()));
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("rms_norm_ext", &rms_norm_ext);
+  m.def("post_norm_residual", &post_norm_residual);
+  m.def("gated_act", &gated_act);
+  m.def("route_sigmoid_topk", &route_sigmoid_topk);
+  m.def("gather_scaled", &gather_scaled);
+  m.def("combine_sum", &combine_sum);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("latent_attn", &latent_attn);
+  m.def("moe_align", &moe_align);
+}

@@ -1,0 +1,68 @@
+// Host launchers of the dtype-generic kernels (bf16 or fp32 storage, fp32 arithmetic): sublayer-output
+// norms into an fp32 residual stream, gated activations, sigmoid top-k routing with input-scaled experts,
+// and latent (compressed-KV) attention with a sliding window and a softmax sink. Raw pointers + an explicit
+// stream, no allocation and no synchronisation: every launcher is hipGraph-capturable. `f32` selects the
+// storage type of the activation / cache / weight tensors (false: bf16).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace die {
+
+// out[r] = x[r] / sqrt(mean(x[r]^2) + eps) * (w or 1 + w); in_f32 / out_f32 / w_f32 give each tensor's storage
+hipError_t launch_rms_norm_ext(void* out, int64_t ostride, bool out_f32, const void* x, int64_t xstride, bool in_f32,
+                               const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
+                               hipStream_t s);
+// resid[r] (fp32) += y[r] / sqrt(mean(y[r]^2) + eps) * (w or 1 + w); act[r] (optional, bf16) = resid[r]
+hipError_t launch_post_norm_residual(float* resid, void* act, const void* y, int64_t ystride, bool y_f32,
+                                     const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
+                                     hipStream_t s);
+// out[r, :f] = act(gu[r, :f]) * f(gu[r, f:2f]).  kind 0: silu(g) * u.  kind 1: g' = min(g, limit),
+// u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1)
+hipError_t launch_gated_act(void* out, const void* gu, bool f32, int rows, int f, int kind, float limit, float alpha,
+                            hipStream_t s);
+
+// Router: z = x . Wr[e] in fp32, score = sigmoid(z), the K largest per token (lowest index on ties);
+// w [T, K] fp32 = the chosen scores (not renormalised), ids [T, K] int32
+hipError_t launch_route_sigmoid_topk(float* w, int* ids, const void* x, int64_t xstride, bool x_f32, const void* wr,
+                                     bool wr_f32, int T, int H, int E, int K, hipStream_t s);
+// xs[j] = w[sorted[j]] * x[sorted[j] / K]  (sorted == nullptr: j itself)
+hipError_t launch_gather_scaled(void* xs, const void* x, bool f32, const int* sorted, const float* w, int n, int K,
+                                int H, hipStream_t s);
+// out[t] (fp32) = sum_k ys[pos[t * K + k]] (+ extra[t]);  pos == nullptr: t * K + k
+hipError_t launch_combine_sum(float* out, const void* ys, bool f32, const int* pos, const void* extra, int T, int K,
+                              int H, hipStream_t s);
+
+struct LatentShape {
+  int rank;      // latent (compressed KV) width, normalised
+  int rot_dim;   // shared rotary key width, stored after the latent
+  int rot_pairs; // rotated pairs (2i, 2i + 1), i < rot_pairs <= rot_dim / 2; the rest passes unchanged
+  const float* inv_freq;  // [rot_pairs] fp32 (device): the angle of pair i at position p is p * inv_freq[i]
+};
+// cache row of token t (at slot_mapping[t] >= 0): [ rmsnorm(kv[t, :rank]) * w | rotate(kv[t, rank:]) ]
+hipError_t launch_latent_kv_write(void* cache, const void* kv, int64_t kvstride, bool f32, const void* w, bool w_f32,
+                                  const int64_t* positions, const int64_t* slots, int T, LatentShape sh, float eps,
+                                  hipStream_t s);
+
+struct LatentAttnArgs {
+  void* out;              // [H, T, rank] latent-space attention output
+  const void* q_lat;      // [H, T, rank] queries projected into the latent space
+  const void* q_rot;      // rotary part of the queries: row t, head h at q_rot + t * q_stride + h * q_hstride
+  int64_t q_stride, q_hstride;
+  const void* cache;      // [num_blocks, block_size, rank + rot_dim]
+  const int* block_tables;
+  int bt_stride;
+  const int* cu_q;        // [S + 1] first row of each sequence (nullptr: one row per sequence)
+  const int* ctx_lens;    // [S] keys after this step
+  const int64_t* positions;
+  const float* sink;      // [H] or nullptr
+  int num_seqs, total_q, max_q, heads, block_size;
+  int window;             // keys j with 0 <= p - j < window (0: all j <= p)
+  float scale;
+  LatentShape sh;
+  bool f32;
+};
+hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s);
+
+}  // namespace die

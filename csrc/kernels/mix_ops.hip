@@ -1,0 +1,236 @@
+// Dtype-generic elementwise / normalisation / routing kernels (gfx950). Storage is bf16 or fp32, selected per
+// tensor at run time; every value is widened to fp32 on load and all arithmetic (sums of squares, norms,
+// sigmoids, router dot products, the residual sum) is fp32. One workgroup per row; rows of any width.
+//
+//   rms_norm_ext          y = x / sqrt(mean(x^2) + eps) * (w | 1 + w)
+//   post_norm_residual    resid(fp32) += rmsnorm(y) * (w | 1 + w); optional bf16 copy of the new residual
+//   gated_act             silu(g) * u, or the clamped variant g' * sigmoid(alpha g') * (u' + 1)
+//   route_sigmoid_topk    router logits (fp32), sigmoid scores, top-K without renormalisation
+//   gather_scaled         expert input rows scaled by their routing weight
+//   combine_sum           per-token sum of its experts' outputs (+ a shared expert), fp32
+//   latent_kv_write       compressed-KV cache row: normalised latent | rotated shared key part
+#include "common.h"
+#include "mix_launchers.h"
+
+namespace die {
+
+namespace {
+
+__device__ __forceinline__ float ldv(const void* p, int64_t i, bool f32) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ void stv(void* p, int64_t i, bool f32, float v) {
+  if (f32)
+    reinterpret_cast<float*>(p)[i] = v;
+  else
+    reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
+}
+
+constexpr int NT = 256;
+
+__device__ __forceinline__ float row_rs(const void* x, int64_t base, bool f32, int n, float eps, float* red) {
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += NT) {
+    const float v = ldv(x, base + c, f32);
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  return 1.0f / sqrtf(ss / (float)n + eps);
+}
+
+__global__ void __launch_bounds__(NT) rms_norm_ext_kernel(void* out, int64_t ostride, bool out_f32, const void* x,
+                                                         int64_t xstride, bool in_f32, const void* w, bool w_f32,
+                                                         bool unit, float eps, int n) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  const float rs = row_rs(x, r * xstride, in_f32, n, eps, red);
+  for (int c = threadIdx.x; c < n; c += NT) {
+    float g = w ? ldv(w, c, w_f32) : 1.0f;
+    if (unit) g += 1.0f;
+    stv(out, r * ostride + c, out_f32, ldv(x, r * xstride + c, in_f32) * rs * g);
+  }
+}
+
+__global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, void* act, const void* y,
+                                                               int64_t ystride, bool y_f32, const void* w, bool w_f32,
+                                                               bool unit, float eps, int n) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  const float rs = row_rs(y, r * ystride, y_f32, n, eps, red);
+  for (int c = threadIdx.x; c < n; c += NT) {
+    float g = w ? ldv(w, c, w_f32) : 1.0f;
+    if (unit) g += 1.0f;
+    const float v = resid[r * n + c] + ldv(y, r * ystride + c, y_f32) * rs * g;
+    resid[r * n + c] = v;
+    if (act) reinterpret_cast<bf16_t*>(act)[r * n + c] = f2bf(v);
+  }
+}
+
+__global__ void __launch_bounds__(NT) gated_act_kernel(void* out, const void* gu, bool f32, int f, int kind,
+                                                      float limit, float alpha) {
+  const int64_t r = blockIdx.x;
+  for (int c = threadIdx.x; c < f; c += NT) {
+    float g = ldv(gu, r * 2 * f + c, f32), u = ldv(gu, r * 2 * f + f + c, f32), v;
+    if (kind == 0) {
+      v = g / (1.0f + expf(-g)) * u;
+    } else {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      v = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
+    stv(out, r * f + c, f32, v);
+  }
+}
+
+constexpr int ROUTE_E_MAX = 256;
+
+// One workgroup per token: wave v computes the logits of experts v, v + 4, ...; thread 0 selects.
+__global__ void __launch_bounds__(NT) route_sigmoid_topk_kernel(float* w_out, int* id_out, const void* x,
+                                                               int64_t xstride, bool x_f32, const void* wr,
+                                                               bool wr_f32, int H, int E, int K) {
+  __shared__ float z[ROUTE_E_MAX];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < E; e += NT / 64) {
+    float a = 0.f;
+    for (int c = lane; c < H; c += 64) a += ldv(x, (int64_t)t * xstride + c, x_f32) * ldv(wr, (int64_t)e * H + c, wr_f32);
+    a = wave_sum(a);
+    if (lane == 0) z[e] = a;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  for (int k = 0; k < K; ++k) {
+    int bi = -1;
+    float bv = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float v = z[e];
+      if (v != v || v == -INFINITY) continue;  // taken (marked below) or unusable
+      if (bi < 0 || v > bv) {
+        bv = v;
+        bi = e;
+      }
+    }
+    if (bi < 0) bi = 0;
+    w_out[(int64_t)t * K + k] = 1.0f / (1.0f + expf(-bv));
+    id_out[(int64_t)t * K + k] = bi;
+    z[bi] = -INFINITY;
+  }
+}
+
+__global__ void __launch_bounds__(NT) gather_scaled_kernel(void* xs, const void* x, bool f32, const int* sorted,
+                                                          const float* w, int K, int H) {
+  const int64_t j = blockIdx.x;
+  const int flat = sorted ? sorted[j] : (int)j;
+  const int64_t t = flat / K;
+  const float wk = w[flat];
+  for (int c = threadIdx.x; c < H; c += NT) stv(xs, j * H + c, f32, wk * ldv(x, t * H + c, f32));
+}
+
+__global__ void __launch_bounds__(NT) combine_sum_kernel(float* out, const void* ys, bool f32, const int* pos,
+                                                        const void* extra, int K, int H) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += NT) {
+    float a = extra ? ldv(extra, t * H + c, f32) : 0.f;
+    for (int k = 0; k < K; ++k) {
+      const int64_t j = pos ? pos[t * K + k] : t * K + k;
+      a += ldv(ys, j * H + c, f32);
+    }
+    out[t * H + c] = a;
+  }
+}
+
+__global__ void __launch_bounds__(NT) latent_kv_write_kernel(void* cache, const void* kv, int64_t kvstride, bool f32,
+                                                            const void* w, bool w_f32, const int64_t* positions,
+                                                            const int64_t* slots, LatentShape sh, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const int64_t slot = slots[t];
+  if (slot < 0) return;  // uniform per workgroup
+  const int64_t src = t * kvstride, dst = slot * (int64_t)(sh.rank + sh.rot_dim);
+  const float rs = row_rs(kv, src, f32, sh.rank, eps, red);
+  for (int c = threadIdx.x; c < sh.rank; c += NT)
+    stv(cache, dst + c, f32, ldv(kv, src + c, f32) * rs * (w ? ldv(w, c, w_f32) : 1.0f));
+  const float p = (float)positions[t];
+  for (int i = threadIdx.x; i < sh.rot_dim / 2 + (sh.rot_dim & 1); i += NT) {
+    const int c0 = 2 * i;
+    const float u = ldv(kv, src + sh.rank + c0, f32);
+    if (c0 + 1 >= sh.rot_dim) {
+      stv(cache, dst + sh.rank + c0, f32, u);
+      continue;
+    }
+    const float v = ldv(kv, src + sh.rank + c0 + 1, f32);
+    if (i < sh.rot_pairs) {
+      float sn, cs;
+      sincosf(p * sh.inv_freq[i], &sn, &cs);
+      stv(cache, dst + sh.rank + c0, f32, u * cs - v * sn);
+      stv(cache, dst + sh.rank + c0 + 1, f32, v * cs + u * sn);
+    } else {
+      stv(cache, dst + sh.rank + c0, f32, u);
+      stv(cache, dst + sh.rank + c0 + 1, f32, v);
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_rms_norm_ext(void* out, int64_t ostride, bool out_f32, const void* x, int64_t xstride, bool in_f32,
+                               const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
+                               hipStream_t s) {
+  if (rows == 0) return hipSuccess;
+  if (n <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(rms_norm_ext_kernel, dim3(rows), dim3(NT), 0, s, out, ostride, out_f32, x, xstride, in_f32, w,
+                     w_f32, unit_offset, eps, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_post_norm_residual(float* resid, void* act, const void* y, int64_t ystride, bool y_f32,
+                                     const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
+                                     hipStream_t s) {
+  if (rows == 0) return hipSuccess;
+  if (n <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(post_norm_residual_kernel, dim3(rows), dim3(NT), 0, s, resid, act, y, ystride, y_f32, w, w_f32,
+                     unit_offset, eps, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_gated_act(void* out, const void* gu, bool f32, int rows, int f, int kind, float limit, float alpha,
+                            hipStream_t s) {
+  if (rows == 0) return hipSuccess;
+  if (f <= 0 || kind < 0 || kind > 1) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(gated_act_kernel, dim3(rows), dim3(NT), 0, s, out, gu, f32, f, kind, limit, alpha);
+  return hipGetLastError();
+}
+
+hipError_t launch_route_sigmoid_topk(float* w, int* ids, const void* x, int64_t xstride, bool x_f32, const void* wr,
+                                     bool wr_f32, int T, int H, int E, int K, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(T), dim3(NT), 0, s, w, ids, x, xstride, x_f32, wr, wr_f32, H, E,
+                     K);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_scaled(void* xs, const void* x, bool f32, const int* sorted, const float* w, int n, int K,
+                                int H, hipStream_t s) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(gather_scaled_kernel, dim3(n), dim3(NT), 0, s, xs, x, f32, sorted, w, K, H);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_sum(float* out, const void* ys, bool f32, const int* pos, const void* extra, int T, int K,
+                              int H, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  hipLaunchKernelGGL(combine_sum_kernel, dim3(T), dim3(NT), 0, s, out, ys, f32, pos, extra, K, H);
+  return hipGetLastError();
+}
+
+hipError_t launch_latent_kv_write(void* cache, const void* kv, int64_t kvstride, bool f32, const void* w, bool w_f32,
+                                  const int64_t* positions, const int64_t* slots, int T, LatentShape sh, float eps,
+                                  hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (sh.rank <= 0 || sh.rot_dim < 0 || sh.rot_pairs * 2 > sh.rot_dim) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(latent_kv_write_kernel, dim3(T), dim3(NT), 0, s, cache, kv, kvstride, f32, w, w_f32, positions,
+                     slots, sh, eps);
+  return hipGetLastError();
+}
+
+}  // namespace die

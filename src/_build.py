@@ -95,6 +95,52 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
     return out
 
 
+MIX_KERNELS = ["mix_ops", "latent_attn", "moe"]
+# hipcc only: keeps -O3 from forming packed fp32 instructions out of ordinary float code
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_mix(force: bool = False, jobs: int = 8, verbose: bool = False) -> str:
+    """``src/_Cmix*.so``: the dtype-generic kernels (post-norm residual, gated activations, sigmoid routing,
+    latent attention) and their bindings — a small extension of its own, so a model that runs on these
+    alone compiles these alone."""
+    odir = os.path.join(OBJ, "mix")
+    os.makedirs(odir, exist_ok=True)
+    out = os.path.join(ROOT, "src", "_Cmix" + EXT_SUFFIX)
+    kdir = os.path.join(CSRC, "kernels")
+    hdrs = _headers(kdir)
+    incs, torch_lib, abi = _torch_paths()
+    jobs_list, objs = [], []
+    for k in MIX_KERNELS:
+        src = os.path.join(kdir, k + ".hip")
+        obj = os.path.join(odir, k + ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + hdrs + [os.path.abspath(__file__)]):
+            jobs_list.append([HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", *NO_PACKED_FP32, "-I",
+                              CSRC, "-c", src, "-o", obj])
+    bsrc = os.path.join(CSRC, "bindings_mix.cpp")
+    bobj = os.path.join(odir, "bindings_mix.o")
+    objs.append(bobj)
+    if force or _newer(bobj, [bsrc] + hdrs):
+        cmd = ["g++", "-O2", "-std=c++17", "-fPIC",
+               f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1",
+               "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_Cmix", "-DTORCH_API_INCLUDE_EXTENSION_H",
+               "-I", CSRC, "-I", "/opt/rocm/include", "-I", sysconfig.get_paths()["include"]]
+        for i in incs:
+            cmd += ["-isystem", i]
+        cmd += ["-c", bsrc, "-o", bobj]
+        jobs_list.append(cmd)
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for res in ex.map(_run, jobs_list):
+            if verbose and res:
+                print(res)
+    if force or _newer(out, objs + [os.path.abspath(__file__)]):
+        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", out,
+              "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+              f"-Wl,-rpath,{torch_lib}"])
+    return out
+
+
 def build_runtime(force: bool = False) -> str:
     out = os.path.join(ROOT, "src", "_runtime" + EXT_SUFFIX)
     rdir = os.path.join(CSRC, "runtime")
@@ -111,17 +157,22 @@ def build_runtime(force: bool = False) -> str:
 def build_all(force: bool = False, verbose: bool = False) -> None:
     build_runtime(force)
     build_kernels(force, verbose=verbose)
+    build_mix(force, verbose=verbose)
 
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
     ap.add_argument("--runtime-only", action="store_true")
+    ap.add_argument("--mix-only", action="store_true", help="the host runtime and src/_Cmix only")
     ap.add_argument("-v", "--verbose", action="store_true")
     a = ap.parse_args(argv)
     print(build_runtime(a.force))
-    if not a.runtime_only:
+    if a.mix_only:
+        print(build_mix(a.force, verbose=a.verbose))
+    elif not a.runtime_only:
         print(build_kernels(a.force, verbose=a.verbose))
+        print(build_mix(a.force, verbose=a.verbose))
     return 0
 
 

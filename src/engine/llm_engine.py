@@ -39,10 +39,14 @@ logger = logging.getLogger(__name__)
 def plan_kv_blocks(arch: ArchConfig, model: CausalLM, cfg: EngineConfig, device: torch.device) -> int:
     if cfg.num_kv_blocks:
         return cfg.num_kv_blocks
-    per_block = KVPool.bytes_per_block(arch.num_layers, model.hkv, cfg.block_size, arch.head_dim)
     if device.type != "cuda":
         return 512
     free, total = torch.cuda.mem_get_info(device)
+    if hasattr(model, "kv_bytes_per_block"):  # a model with its own cache layout prices its blocks and activations
+        act = model.activation_bytes(cfg.max_num_batched_tokens) + cfg.max_num_seqs * arch.vocab_size * 4
+        budget = min(free - act, cfg.gpu_memory_fraction * total - (total - free) - act)
+        return max(16, int(budget // model.kv_bytes_per_block(cfg.block_size)))
+    per_block = KVPool.bytes_per_block(arch.num_layers, model.hkv, cfg.block_size, arch.head_dim)
     h = arch.hidden_size
     inter = model.inter * (arch.top_k if arch.is_moe else 1)
     t = cfg.max_num_batched_tokens
@@ -102,15 +106,21 @@ class LLMEngine:
         if hasattr(model, "pack_lm_head"):
             model.pack_lm_head()
         nblocks = plan_kv_blocks(self.arch, model, cfg, self.device)
-        self.pool = KVPool(self.arch.num_layers, nblocks, model.hkv, cfg.block_size, self.arch.head_dim,
-                           self.device, dtype=model.dtype)
+        if hasattr(model, "make_kv_pool"):  # the model's own cache layout (e.g. one latent row per token and layer)
+            self.pool = model.make_kv_pool(nblocks, cfg.block_size)
+            per_block = model.kv_bytes_per_block(cfg.block_size)
+            can_move = getattr(self.pool, "uniform", True) and model.dtype == torch.bfloat16
+        else:
+            self.pool = KVPool(self.arch.num_layers, nblocks, model.hkv, cfg.block_size, self.arch.head_dim,
+                               self.device, dtype=model.dtype)
+            per_block = KVPool.bytes_per_block(self.arch.num_layers, model.hkv, cfg.block_size, self.arch.head_dim)
+            can_move = True
         self.blocks = KVBlockManager(nblocks, cfg.block_size, cfg.enable_prefix_caching, cfg.kv_block_ttl_s)
         self.runner = runner_cls(model, self.pool, cfg, self.max_model_len)
         # host swap space for preempted sequences (single-process runners only: a TP group would
         # have to mirror every swap on its followers, so it always recomputes)
-        per_block = KVPool.bytes_per_block(self.arch.num_layers, model.hkv, cfg.block_size, self.arch.head_dim)
         swap_blocks = 0
-        if cfg.preemption_mode != "recompute" and getattr(self.runner, "supports_swap", False):
+        if cfg.preemption_mode != "recompute" and getattr(self.runner, "supports_swap", False) and can_move:
             swap_blocks = int(cfg.swap_space_gib * 2**30 // per_block)
         self.scheduler = Scheduler(cfg, self.blocks, self.max_model_len, swap_capacity_blocks=swap_blocks)
         self.seqs: Dict[str, Sequence] = {}
@@ -147,12 +157,14 @@ class LLMEngine:
     def from_pretrained(cls, path: str, device="cuda:0", cfg: Optional[EngineConfig] = None,
                         max_model_len: int = 4096, tp: Optional[TPContext] = None, capture: bool = True,
                         dtype=torch.bfloat16, **arch_overrides):
-        """A local HF-format checkpoint directory (config.json + *.safetensors)."""
-        from src.models.loader import arch_from_hf_config, load_checkpoint
+        """A local checkpoint directory (config.json + *.safetensors) of any registered model family."""
+        from src.models.loader import load_checkpoint
+        from src.models.registry import resolve
 
-        arch = arch_from_hf_config(path, **arch_overrides)
+        # the model class is chosen by config.json (src/models/registry.py)
+        _, arch, model_cls = resolve(path, **arch_overrides)
         cfg = cfg or EngineConfig()
-        model = CausalLM(arch, device, dtype=dtype, tp=tp, max_position=max(max_model_len, 16))
+        model = model_cls(arch, device, dtype=dtype, tp=tp, max_position=max(max_model_len, 16))
         load_checkpoint(model, path)
         eng = cls(model, cfg, max_model_len)
         if capture:
@@ -554,6 +566,44 @@ class LLMEngine:
             seq._preempted_outputs = []  # type: ignore[attr-defined]
         if seq.on_finish is not None:
             seq.on_finish(seq)
+
+    # --------------------------------------------------------------- replay
+    def replay_step(self, entries, end=()) -> torch.Tensor:
+        """One teacher-forced engine step. ``entries``: (request id, its next token ids, wanted places among
+        them) per request, all run together as one batch from the cache that earlier steps left; a request is
+        admitted at its first entry and may sit out any step. ``end``: requests finished after this step (their
+        blocks go back to the pool). Returns the fp32 logits at the wanted places, in entry order, [n, vocab]
+        on the host. Nothing is sampled; the scheduler, block manager, runner and kernels are the serving ones."""
+        plan, rows, base = [], [], 0
+        for rid, toks, want in entries:
+            toks = [int(x) for x in toks]
+            if toks and (min(toks) < 0 or max(toks) >= self.arch.vocab_size):
+                raise ValueError(f"token id outside [0, {self.arch.vocab_size})")
+            seq = self.seqs.get(rid)
+            if seq is None:
+                seq = Sequence(rid, [], SamplingParams(max_tokens=1))
+                self.seqs[rid] = seq
+                self.scheduler.add(seq)
+            seq.prompt_ids.extend(toks)
+            self.stats["prompt_tokens"] += len(toks)
+            plan.append((seq, len(toks)))
+            for w in want:
+                if not 0 <= int(w) < len(toks):
+                    raise ValueError(f"{rid}: wanted place {w} outside the step's {len(toks)} tokens")
+                rows.append(base + int(w))
+            base += len(toks)
+        out = self.scheduler.schedule_forced(plan)
+        logits = self.runner.forward_logits(out.prefill, rows) if out.prefill else \
+            torch.empty(0, self.arch.vocab_size, dtype=torch.float32)
+        for c in out.prefill:
+            c.seq.num_computed = c.start + c.length
+        for rid in end:
+            seq = self.seqs.pop(rid, None)
+            if seq is not None:
+                self.scheduler.finish(seq, "replay_end")
+                self.stats["finished"] += 1
+        self.stats["steps"] += 1
+        return logits
 
     # ------------------------------------------------------------- helpers
     def generate(self, prompts: List[List[int]], sampling: SamplingParams) -> List[List[int]]:

@@ -130,7 +130,7 @@ class ModelRunner:
         self.d_tokens = torch.zeros(2 * self.k_max, self.max_seqs, dtype=i64, device=dev)
         self.d_ctl = torch.zeros(2, dtype=i32, device=dev)
         self.d_adv_ticket = torch.zeros(1, dtype=i32, device=dev)  # sample_advance's row ticket (re-armed in-kernel)
-        if self.is_cuda:
+        if self.is_cuda and getattr(model, "needs_decode_partials", True):
             maxp = ops.decode_partials(max_model_len)
             hq = model.hq
             self.part_o = torch.empty(self.max_seqs * hq * maxp * 128, dtype=torch.float32, device=dev)
@@ -147,7 +147,7 @@ class ModelRunner:
         self.supports_swap = type(self)._sync_step is ModelRunner._sync_step
         # a runner whose steps are mirrored by other ranks (tensor parallelism) must mirror whole windows too:
         # it declares that with mirrors_windows (TPModelRunner sends one message per window, not per step)
-        self.supports_multistep = self.is_cuda and self.k_max > 1 and (
+        self.supports_multistep = self.is_cuda and self.k_max > 1 and ops.native_available() and (
             type(self)._sync_step is ModelRunner._sync_step or self.mirrors_windows)
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self.graph_sizes: List[int] = []
@@ -242,14 +242,8 @@ class ModelRunner:
         """Run one ragged prefill batch — or a mixed step, whose decode rows are 1-token chunks —
         and return the sampled token for every chunk that completes its prompt or decodes
         (None for partial prompt chunks)."""
-        toks = [c.tokens() for c in chunks]
-        starts = [c.start for c in chunks]
-        tables = [c.seq.block_table for c in chunks]
         n = len(chunks)
-        t = self.rt.build_prefill_inputs(toks, starts, tables, self.bs, self.h_ids.data_ptr(),
-                                         self.h_pos.data_ptr(), self.h_slots.data_ptr(), self.h_cu.data_ptr(),
-                                         self.h_ctx.data_ptr(), self.h_bt.data_ptr(), self.bt_width,
-                                         self.h_last.data_ptr())
+        t = self._stage_chunks(chunks)
         done = [i for i, c in enumerate(chunks) if c.completes_prompt]
         nd = len(done)
         if nd and nd != n:
@@ -270,6 +264,43 @@ class ModelRunner:
             torch.cuda.current_stream(self.device).synchronize()
             self._raise_on_fault()
         return res
+
+    def _stage_chunks(self, chunks: List[PrefillChunk]) -> int:
+        """A ragged batch's inputs (ids, positions, KV slots, row offsets, context lengths, block tables, last
+        rows) into the pinned staging buffers, by the native step builder. Returns the number of rows."""
+        return self.rt.build_prefill_inputs([c.tokens() for c in chunks], [c.start for c in chunks],
+                                            [c.seq.block_table for c in chunks], self.bs, self.h_ids.data_ptr(),
+                                            self.h_pos.data_ptr(), self.h_slots.data_ptr(), self.h_cu.data_ptr(),
+                                            self.h_ctx.data_ptr(), self.h_bt.data_ptr(), self.bt_width,
+                                            self.h_last.data_ptr())
+
+    @torch.inference_mode()
+    def forward_logits(self, chunks: List[PrefillChunk], rows: List[int]) -> torch.Tensor:
+        """Teacher-forced step: run one ragged batch (prompt portions beside single decode tokens) through the
+        same staging, cache writes and kernels as :meth:`prefill` / :meth:`decode`, sample nothing, and return
+        the fp32 logits [len(rows), vocab] at the given rows of the batch (row = index into the concatenated
+        chunk tokens). A batch of single tokens runs the decode form of the step (one query row per sequence)."""
+        n = len(chunks)
+        t = self._stage_chunks(chunks)
+        self._h2d(t, n, with_cu=True)
+        dev = self.device
+        single = all(c.length == 1 for c in chunks)
+        if single:
+            meta = AttnMetadata(is_prefill=False, slot_mapping=self.d_slots[:n], block_tables=self.d_bt[:n],
+                                ctx_lens=self.d_ctx[:n], max_ctx=self.max_model_len, part_o=self.part_o,
+                                part_ml=self.part_ml, attn_cnt=self.attn_cnt)
+        else:
+            meta = AttnMetadata(is_prefill=True, slot_mapping=self.d_slots[:t], block_tables=self.d_bt[:n],
+                                ctx_lens=self.d_ctx[:n], cu_q=self.d_cu[: n + 1],
+                                max_q_len=max(c.length for c in chunks))
+        hidden = self.model.forward(self.d_ids[:t], self.d_pos[:t], meta, self.pool.tensor)
+        if not rows:
+            if self.is_cuda:
+                torch.cuda.current_stream(dev).synchronize()
+            return torch.empty(0, self.model.arch.vocab_size, dtype=torch.float32)
+        sel = torch.tensor(rows, dtype=torch.int64).to(dev, non_blocking=False)
+        logits = self.model.compute_logits(hidden.index_select(0, sel)).float()
+        return logits.cpu()
 
     def _exec_prefill(self, t: int, n: int, max_q: int, nd: int, greedy: bool, kv_hook=None) -> Optional[torch.Tensor]:
         # the last layer runs only for the sampled rows (CausalLM._last_layer_kept_rows; DIE_PRUNE_LAST=0: all)

@@ -258,6 +258,38 @@ class Scheduler:
             self.steps_decode += 1
         return out
 
+    def schedule_forced(self, plan: List[Tuple[Sequence, int]]) -> SchedulerOutput:
+        """A teacher-forced step: exactly these (sequence, number of its next tokens) pairs run, in this order,
+        as one ragged batch — prompt portions of any length beside single tokens. New sequences are admitted
+        (waiting -> running), every sequence's block table grows to hold its new tokens, and nothing is
+        preempted: a step that does not fit the KV pool or the sequence limit is an error of the caller's plan."""
+        out = SchedulerOutput()
+        for seq, n in plan:
+            if n <= 0:
+                raise ValueError(f"{seq.request_id}: a forced step needs at least one token")
+            if seq.status == SeqStatus.WAITING:
+                if seq in self.waiting:
+                    self.waiting.remove(seq)
+                if len(self.running) >= self.cfg.max_num_seqs:
+                    raise RuntimeError(f"more than max_num_seqs={self.cfg.max_num_seqs} live sequences")
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+            elif seq.status != SeqStatus.RUNNING:
+                raise RuntimeError(f"{seq.request_id}: not live")
+            if seq.num_computed + n > self.max_model_len:
+                raise RuntimeError(f"{seq.request_id}: exceeds max_model_len={self.max_model_len}")
+            if not self.blocks.ensure_slots(seq, seq.num_computed + n):
+                raise RuntimeError("KV pool exhausted by a forced step")
+            out.prefill.append(PrefillChunk(seq, seq.num_computed, n))
+        if out.prefill:
+            if all(c.length == 1 and c.start > 0 for c in out.prefill):
+                self.steps_decode += 1
+            elif any(c.length == 1 and c.start > 0 for c in out.prefill):
+                self.steps_mixed += 1
+            else:
+                self.steps_prefill += 1
+        return out
+
     def _defer_prefill(self, now: float, blocked: bool) -> bool:
         """Hold newly arrived prompts while sequences decode (cfg.prefill_batch_tokens): True while
         fewer than that many prompt tokens wait and the oldest is younger than prefill_batch_wait_ms.

@@ -917,3 +917,8 @@ def _moe_decode_tiles(hdim: int, inter: int, t: int):
 
 def _moe_down_wr(hdim: int, inter: int) -> int:
     return 64 if hdim % 64 == 0 else 32
+
+
+# dtype-generic ops (bf16 / fp32 storage) of the src/_Cmix extension
+from .mix import (ACT_CLAMPED, ACT_SILU, gated_act, latent_attn, latent_kv_write, mix_available,  # noqa: E402,F401
+                  moe_input_scaled, post_norm_residual, rms_norm_ext, rope_inv_freq, route_sigmoid_topk)

@@ -1,0 +1,170 @@
+"""
+Dtype-generic ops (bf16 or fp32 storage, fp32 arithmetic) on the ``src/_Cmix`` HIP extension:
+
+* :func:`rms_norm_ext`, :func:`post_norm_residual` — RMS norms with a plain or a stored-around-zero weight,
+  the second one applied to a sublayer's OUTPUT and added into an fp32 residual stream;
+* :func:`gated_act` — SiLU-gated and clamped sigmoid-gated feed-forward activations;
+* :func:`route_sigmoid_topk`, :func:`moe_input_scaled` — sigmoid-scored top-k routing whose weight scales
+  the expert's input, with an optional always-on shared expert;
+* :func:`latent_kv_write`, :func:`latent_attn` — latent (compressed-KV) attention over a paged cache of
+  [latent | rotated shared key] rows, with a sliding window and a per-head softmax sink.
+
+GPU tensors always run the HIP kernels (a missing extension raises); CPU tensors run the plain-PyTorch
+semantics in :mod:`src.ops.reference`, which lets the engine's control flow run in CPU-only tests.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from . import reference as ref
+
+_Cmix = None
+_CMIX_ERR: Optional[BaseException] = None
+try:
+    from src import _Cmix  # type: ignore  # noqa: F811
+except Exception as e:  # pragma: no cover - depends on build state
+    _CMIX_ERR = e
+
+
+def mix_available() -> bool:
+    return _Cmix is not None
+
+
+def _kern():
+    if _Cmix is None:
+        raise RuntimeError(
+            "HIP kernel extension src/_Cmix is not built or failed to load "
+            f"({_CMIX_ERR!r}); run `python -m src._build --mix-only` (hipcc --offload-arch=gfx950)")
+    return _Cmix
+
+
+def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_offset: bool = False,
+                 out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * g over the last dim of [rows, n] (any row stride); g = w, or 1 + w with
+    ``unit_offset`` (a weight stored around zero), or 1 without a weight."""
+    out_dtype = out_dtype or x.dtype
+    if not x.is_cuda:
+        return ref.rms_norm_ext(x, w, eps, unit_offset).to(out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _kern().rms_norm_ext(out, x, w, unit_offset, eps)
+    return out
+
+
+def post_norm_residual(resid: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float, unit_offset: bool = True,
+                       act: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """resid (fp32 [rows, n], in place) += rmsnorm(y) * g — the norm sits on the sublayer's output, the residual
+    sum is fp32. ``act`` (bf16, same shape): also receives the new residual, the next projection's input."""
+    if not resid.is_cuda:
+        resid.add_(ref.rms_norm_ext(y, w, eps, unit_offset).float())
+        if act is not None:
+            act.copy_(resid)
+        return resid
+    _kern().post_norm_residual(resid, act, y, w, unit_offset, eps)
+    return resid
+
+
+ACT_SILU, ACT_CLAMPED = 0, 1
+
+
+def gated_act(gu: torch.Tensor, kind: int = ACT_SILU, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """[rows, 2f] = [gate | up] -> [rows, f]. ACT_SILU: silu(g) * u. ACT_CLAMPED: g' = min(g, limit),
+    u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1)."""
+    if not gu.is_cuda:
+        return ref.gated_act(gu, kind, limit, alpha)
+    gu = gu.contiguous()
+    out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+    _kern().gated_act(out, gu, kind, limit, alpha)
+    return out
+
+
+def route_sigmoid_topk(x: torch.Tensor, router: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(w [T, k] fp32, ids [T, k] int32): the k experts with the largest sigmoid(x . router[e]) (fp32 logits) and
+    those scores, not renormalised."""
+    if not x.is_cuda:
+        return ref.route_sigmoid_topk(x, router, k)
+    t = x.shape[0]
+    w = torch.empty(t, k, dtype=torch.float32, device=x.device)
+    ids = torch.empty(t, k, dtype=torch.int32, device=x.device)
+    _kern().route_sigmoid_topk(w, ids, x, router.contiguous())
+    return w, ids
+
+
+# (token, expert) rows up to which the experts' weights are gathered per row for two batched GEMMs (no host
+# read, hipGraph-capturable: decode steps); above it each expert runs one library GEMM pair over its rows
+MOE_BMM_MAX_ROWS = 64
+
+
+def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: torch.Tensor, ids: torch.Tensor,
+                     extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] (fp32) = sum_j expert_{ids[t, j]}(w[t, j] * x[t]) (+ extra[t]); expert(z) = W2 (silu(W1 z) * (W3 z))
+    with w13 [E, 2f, H] = [W1; W3] and w2 [E, H, f]. The routing weight multiplies the expert's INPUT."""
+    if not x.is_cuda:
+        return ref.moe_input_scaled(x, w13, w2, w, ids, extra)
+    kern = _kern()
+    t, h = x.shape
+    k = ids.shape[1]
+    n = t * k
+    e = w13.shape[0]
+    x = x.contiguous()
+    w = w.contiguous()
+    out = torch.empty(t, h, dtype=torch.float32, device=x.device)
+    xs = torch.empty(n, h, dtype=x.dtype, device=x.device)
+    if n <= MOE_BMM_MAX_ROWS or torch.cuda.is_current_stream_capturing():
+        kern.gather_scaled(xs, x, None, w, k)
+        sel = ids.reshape(-1).long()
+        g = torch.bmm(w13.index_select(0, sel), xs.unsqueeze(2)).squeeze(2)
+        ys = torch.bmm(w2.index_select(0, sel), gated_act(g, ACT_SILU).unsqueeze(2)).squeeze(2).contiguous()
+        kern.combine_sum(out, ys, None, extra, k)
+        return out
+    offsets = torch.empty(e + 1, dtype=torch.int32, device=x.device)
+    sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
+    pos = torch.empty(n, dtype=torch.int32, device=x.device)
+    kern.moe_align(offsets, sorted_idx, pos, ids.reshape(-1).contiguous(), e)
+    kern.gather_scaled(xs, x, sorted_idx, w, k)
+    ys = torch.empty(n, h, dtype=x.dtype, device=x.device)
+    off = offsets.tolist()  # one host read per layer: the per-expert groups become library GEMMs
+    for ei in range(e):
+        a0, a1 = off[ei], off[ei + 1]
+        if a1 > a0:
+            F.linear(gated_act(F.linear(xs[a0:a1], w13[ei]), ACT_SILU), w2[ei], out=ys[a0:a1])
+    kern.combine_sum(out, ys, pos, extra, k)
+    return out
+
+
+def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
+    """fp32 [dims / 2]: base^(-2 i / dims), rounded once from float64."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / dims)).float().to(device)
+
+
+def latent_kv_write(cache: torch.Tensor, kv: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
+                    slots: torch.Tensor, rank: int, rot_dim: int, inv_freq: torch.Tensor, eps: float) -> None:
+    """cache [blocks, block_size, rank + rot_dim]: the row at slot slots[t] (< 0: skipped) becomes
+    [rmsnorm(kv[t, :rank]) * w | kv[t, rank:] with its first 2 * len(inv_freq) dims rotated as interleaved
+    pairs (2i, 2i + 1) by the angle positions[t] * inv_freq[i]]."""
+    if not kv.is_cuda:
+        ref.latent_kv_write(cache, kv, w, positions, slots, rank, rot_dim, inv_freq, eps)
+        return
+    _kern().latent_kv_write(cache, kv, w, positions, slots, rank, rot_dim, inv_freq, eps)
+
+
+def latent_attn(q_lat: torch.Tensor, q: torch.Tensor, rot_off: int, cache: torch.Tensor, block_tables: torch.Tensor,
+                cu_q: Optional[torch.Tensor], ctx_lens: torch.Tensor, positions: torch.Tensor,
+                sink: Optional[torch.Tensor], max_q: int, window: int, scale: float, rot_dim: int,
+                inv_freq: torch.Tensor) -> torch.Tensor:
+    """Absorbed latent attention. q_lat [H, T, rank]: the queries projected into the latent space; q [T, H * qh]:
+    the full queries, head h's rotary part at [h * qh + rot_off, + rot_dim) (rotated here, by positions[t]).
+    Row (t, h) scores the cache rows j of its sequence with 0 <= p - j < window (window 0: j <= p):
+    (q_lat . latent_j + q_rot . krot_j) * scale, softmax with exp(sink[h]) added to the denominator, and
+    returns the weighted sum of the latent rows, [H, T, rank]. cu_q None: one query row per sequence."""
+    if not q_lat.is_cuda:
+        return ref.latent_attn(q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, window, scale,
+                               rot_dim, inv_freq)
+    out = torch.empty_like(q_lat)
+    _kern().latent_attn(out, q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, max_q, window,
+                        scale, rot_dim, inv_freq)
+    return out

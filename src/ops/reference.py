@@ -168,3 +168,101 @@ def moe_experts(x, w13, w2, w, ids):
         y = a.to(x.dtype).float() @ w2[e].float().t()
         out.index_add_(0, tok, y * w[tok, slot][:, None])
     return out.to(x.dtype)
+
+
+# ----------------------------------------------------------------- dtype-generic ops (src/ops/mix.py)
+def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_offset: bool = False) -> torch.Tensor:
+    xf = x.float()
+    y = xf / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        y = y * (w.float() + 1.0 if unit_offset else w.float())
+    return y.to(x.dtype)
+
+
+def gated_act(gu: torch.Tensor, kind: int, limit: float, alpha: float) -> torch.Tensor:
+    f = gu.shape[-1] // 2
+    g, u = gu[..., :f].float(), gu[..., f:].float()
+    if kind == 0:
+        return (g * torch.sigmoid(g) * u).to(gu.dtype)
+    g = torch.clamp(g, max=limit)
+    u = torch.clamp(u, -limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def route_sigmoid_topk(x: torch.Tensor, router: torch.Tensor, k: int):
+    z = x.float() @ router.float().t()
+    zs, ids = torch.sort(z, dim=-1, descending=True, stable=True)
+    return torch.sigmoid(zs[:, :k]).contiguous(), ids[:, :k].to(torch.int32).contiguous()
+
+
+def moe_input_scaled(x, w13, w2, w, ids, extra=None) -> torch.Tensor:
+    t, h = x.shape
+    out = torch.zeros(t, h, dtype=torch.float32) if extra is None else extra.float().clone()
+    for j in range(ids.shape[1]):
+        for e in ids[:, j].unique().tolist():
+            rows = (ids[:, j] == e).nonzero().flatten()
+            xs = (w[rows, j, None] * x[rows].float()).to(x.dtype)
+            a = gated_act(torch.nn.functional.linear(xs, w13[e]), 0, 0.0, 1.0)
+            out[rows] += torch.nn.functional.linear(a, w2[e]).float()
+    return out
+
+
+def _rotate_pairs(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """x [..., n] fp32 with a leading token dim: the first 2 * len(inv_freq) dims rotate as pairs (2i, 2i + 1)."""
+    n = 2 * inv_freq.numel()
+    ang = pos.float().reshape(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    cs, sn = ang.cos(), ang.sin()
+    u, v = x[..., 0:n:2], x[..., 1:n:2]
+    out = x.clone()
+    out[..., 0:n:2] = u * cs - v * sn
+    out[..., 1:n:2] = v * cs + u * sn
+    return out
+
+
+def latent_kv_write(cache, kv, w, positions, slots, rank, rot_dim, inv_freq, eps) -> None:
+    t = kv.shape[0]
+    c = rms_norm_ext(kv[:, :rank], w, eps).float()
+    kr = _rotate_pairs(kv[:, rank:rank + rot_dim].float(), positions[:t], inv_freq)
+    rows = torch.cat([c, kr], -1).to(cache.dtype)
+    flat = cache.view(-1, cache.shape[-1])
+    for i in range(t):
+        s = int(slots[i])
+        if s >= 0:
+            flat[s] = rows[i]
+
+
+def latent_attn(q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, window, scale, rot_dim,
+                inv_freq) -> torch.Tensor:
+    heads, total, rank = q_lat.shape
+    qh = q.shape[1] // heads
+    qr = q.view(total, heads, qh)[:, :, rot_off:rot_off + rot_dim].float()
+    qr = _rotate_pairs(qr, positions[:total], inv_freq)
+    out = torch.zeros(heads, total, rank, dtype=torch.float32)
+    bs = cache.shape[1]
+    nseq = block_tables.shape[0]
+    for s in range(nseq):
+        a, b = (int(cu_q[s]), int(cu_q[s + 1])) if cu_q is not None else (s, s + 1)
+        if b <= a:
+            continue
+        ctx = int(ctx_lens[s])
+        idx = torch.arange(ctx)
+        rows = cache[block_tables[s].long()[idx // bs], idx % bs].float()      # [ctx, rank + rot_dim]
+        p = positions[a:b].long()
+        sc = (torch.einsum("hqr,jr->hqj", q_lat[:, a:b].float(), rows[:, :rank])
+              + torch.einsum("qhd,jd->hqj", qr[a:b], rows[:, rank:])) * scale
+        d = p[:, None] - idx[None, :]
+        ok = d >= 0
+        if window > 0:
+            ok = ok & (d < window)
+        sc = sc.masked_fill(~ok[None], float("-inf"))
+        mx = sc.max(-1).values
+        if sink is not None:
+            mx = torch.maximum(mx, sink.float()[:, None])
+        mx = torch.where(torch.isfinite(mx), mx, torch.zeros_like(mx))
+        e = torch.exp(sc - mx[..., None])
+        den = e.sum(-1)
+        if sink is not None:
+            den = den + torch.exp(sink.float()[:, None] - mx)
+        pr = e / den.clamp_min(1e-38)[..., None]
+        out[:, a:b] = torch.einsum("hqj,jr->hqr", pr, rows[:, :rank])
+    return out.to(q_lat.dtype)
