@@ -212,6 +212,9 @@ def sample(logits, temperature=None, top_k=None, top_p=None, seeds=None, steps=N
         return ref.sample(logits, temperature, top_k, top_p, seeds, steps)
     if out is None:
         out = torch.empty(logits.shape[0], dtype=torch.long, device=logits.device)
+    if logits.dtype != torch.bfloat16 or logits.shape[1] % 8:
+        # the sampling kernel reads bf16 rows of a multiple of 8 columns: padding columns can never be drawn
+        logits = torch.nn.functional.pad(logits.to(torch.bfloat16), (0, -logits.shape[1] % 8), value=float("-inf"))
     part, cnt = scratch if scratch is not None else (None, None)
     _kern().sample(out, logits, temperature, top_k, top_p, seeds, steps, part, cnt, lm_part)
     return out

@@ -48,7 +48,7 @@ def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_of
     ``unit_offset`` (a weight stored around zero), or 1 without a weight."""
     out_dtype = out_dtype or x.dtype
     if not x.is_cuda:
-        return ref.rms_norm_ext(x, w, eps, unit_offset).to(out_dtype)
+        return ref.rms_norm_ext(x, w, eps, unit_offset, out_dtype)
     out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     _kern().rms_norm_ext(out, x, w, unit_offset, eps)
     return out
@@ -59,7 +59,7 @@ def post_norm_residual(resid: torch.Tensor, y: torch.Tensor, w: torch.Tensor, ep
     """resid (fp32 [rows, n], in place) += rmsnorm(y) * g — the norm sits on the sublayer's output, the residual
     sum is fp32. ``act`` (bf16, same shape): also receives the new residual, the next projection's input."""
     if not resid.is_cuda:
-        resid.add_(ref.rms_norm_ext(y, w, eps, unit_offset).float())
+        resid.add_(ref.rms_norm_ext(y, w, eps, unit_offset, torch.float32))
         if act is not None:
             act.copy_(resid)
         return resid

@@ -171,12 +171,13 @@ def moe_experts(x, w13, w2, w, ids):
 
 
 # ----------------------------------------------------------------- dtype-generic ops (src/ops/mix.py)
-def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_offset: bool = False) -> torch.Tensor:
+def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_offset: bool = False,
+                 out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     xf = x.float()
     y = xf / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
     if w is not None:
         y = y * (w.float() + 1.0 if unit_offset else w.float())
-    return y.to(x.dtype)
+    return y.to(out_dtype or x.dtype)
 
 
 def gated_act(gu: torch.Tensor, kind: int, limit: float, alpha: float) -> torch.Tensor:
