@@ -163,7 +163,7 @@ void latent_kv_write(Tensor cache, Tensor kv, Tensor w, Tensor positions, Tensor
 // out, q_lat [H, T, rank]; q [T, H * qh] whose head h keeps its rotary part at [h * qh + rot_off, + rot_dim)
 void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cache, Tensor block_tables,
                  OptTensor cu_q, Tensor ctx_lens, Tensor positions, OptTensor sink, int64_t max_q, int64_t window,
-                 double scale, int64_t rot_dim, Tensor inv_freq) {
+                 double scale, int64_t rot_dim, Tensor inv_freq, int64_t impl) {
   const bool f = is_f32(q_lat, "q_lat");
   TORCH_CHECK(is_f32(out, "out") == f && is_f32(q, "q") == f && is_f32(cache, "cache") == f, "one dtype");
   TORCH_CHECK(q_lat.dim() == 3 && q_lat.is_contiguous() && out.is_contiguous() && out.sizes() == q_lat.sizes(),
@@ -215,6 +215,7 @@ void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cac
   a.scale = (float)scale;
   a.sh = latent_shape(rank, rot_dim, inv_freq);
   a.f32 = f;
+  a.impl = (int)impl;
   HIP_OK(die::launch_latent_attn(a, cur_stream()));
 }
 

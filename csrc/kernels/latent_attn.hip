@@ -166,6 +166,215 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(LatentAttnArgs a, int 
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// bf16 on the matrix cores (v_mfma_f32_32x32x16_bf16), for rank % 32 == 0, rank <= 256, rot_dim % 16 == 0.
+// Workgroup = 4 waves x 32 rows. Per tile of 32 keys, staged once in LDS both row-major (K: [key][Dk]) and
+// transposed (V^T: [d][key'], key' = the key order of the score accumulator's rows, so a PV operand is one
+// 16-byte read):
+//   S^T[key][q] = K Q^T        A = K rows from LDS, B = Q rows from LDS      (Dk / 16 MFMAs)
+//   online softmax per query column (one lane pair owns a query: no cross-lane traffic beyond xor 32),
+//   fp32 scores and weights, running max seeded with the sink; P is rounded to bf16 only as the MFMA operand
+//   O^T[d][q] += V^T P^T      A = V^T from LDS, B = P^T from the accumulator  (2 * rank / 32 MFMAs)
+constexpr int MROWS = 128, MKT = 32, VT_PITCH = 40;  // V^T row pitch in bf16 (80 B: 16-byte aligned reads)
+
+template <int NDB>
+__global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a, int KP) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [MROWS][KP]
+  bf16_t* ks = qs + MROWS * KP;                               // [MKT][KP]
+  bf16_t* vt = ks + MKT * KP;                                 // [32 * NDB][VT_PITCH]
+  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  const int H = a.heads, R = a.sh.rank, Dk = a.sh.rank + a.sh.rot_dim;
+  const int q0 = a.cu_q ? a.cu_q[s] : s;
+  const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
+  const int nrows = nq * H, row0 = blockIdx.x * MROWS;
+  if (row0 >= nrows) return;
+  const int ctx = a.ctx_lens[s];
+  const int last_row = min(row0 + MROWS, nrows) - 1;
+  const int p_first = (int)a.positions[q0 + row0 / H], p_last = (int)a.positions[q0 + last_row / H];
+  const int jlo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  const int jhi = min(p_last, ctx - 1);
+  const bf16_t* qlat = reinterpret_cast<const bf16_t*>(a.q_lat);
+  const bf16_t* qrot = reinterpret_cast<const bf16_t*>(a.q_rot);
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+
+  // queries -> LDS: the latent part as 16-byte copies, the rotary part rotated in fp32
+  const int lch = R / 8;
+  for (int idx = tid; idx < MROWS * lch; idx += 256) {
+    const int r = idx / lch, c = idx % lch, row = row0 + r;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < nrows) {
+      const int64_t t = q0 + row / H;
+      v = *reinterpret_cast<const uint4*>(qlat + ((int64_t)(row % H) * a.total_q + t) * R + 8 * c);
+    }
+    *reinterpret_cast<uint4*>(qs + r * KP + 8 * c) = v;
+  }
+  for (int idx = tid; idx < MROWS * a.sh.rot_dim; idx += 256) {
+    const int r = idx / a.sh.rot_dim, dd = idx % a.sh.rot_dim, row = row0 + r;
+    float v = 0.f;
+    if (row < nrows) {
+      const int64_t t = q0 + row / H;
+      const int64_t qr = t * a.q_stride + (int64_t)(row % H) * a.q_hstride;
+      const int i = dd >> 1;
+      if (i < a.sh.rot_pairs) {
+        const float u = bf2f(qrot[qr + 2 * i]), w = bf2f(qrot[qr + 2 * i + 1]);
+        float sn, cs;
+        sincosf((float)a.positions[t] * a.sh.inv_freq[i], &sn, &cs);
+        v = (dd & 1) ? w * cs + u * sn : u * cs - w * sn;
+      } else {
+        v = bf2f(qrot[qr + dd]);
+      }
+    }
+    qs[r * KP + R + dd] = f2bf(v);
+  }
+
+  const int qcol = lane & 31, hh = lane >> 5;
+  const int myrow = row0 + wave * 32 + qcol;
+  const bool rok = myrow < nrows;
+  const bool wave_live = row0 + wave * 32 < nrows;
+  const int prow = rok ? (int)a.positions[q0 + myrow / H] : -1;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float sl2 = a.scale * LOG2E;
+  const bool has_sink = a.sink != nullptr && rok;
+  float m = has_sink ? a.sink[myrow % H] * LOG2E : -1e30f;
+  float l = has_sink ? 1.0f : 0.0f;
+  f32x16_t o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+
+  const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
+  const int kch = Dk / 8, nkk = Dk / 16;
+  for (int j0 = jlo; j0 <= jhi; j0 += MKT) {
+    __syncthreads();
+    for (int idx = tid; idx < MKT * kch; idx += 256) {
+      const int k = idx / kch, c = idx % kch, j = j0 + k;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (j <= jhi) v = *reinterpret_cast<const uint4*>(
+          cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
+      *reinterpret_cast<uint4*>(ks + k * KP + 8 * c) = v;
+      if (8 * c < R) {
+        const int k16 = k & 15;
+        const int kp = (k & 16) + 8 * ((k16 >> 2) & 1) + (k16 & 3) + 4 * (k16 >> 3);
+        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vt[(8 * c + e) * VT_PITCH + kp] = (bf16_t)((wv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+      }
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+    f32x16_t sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    const bf16_t* ka = ks + qcol * KP + 8 * hh;
+    const bf16_t* qb = qs + (wave * 32 + qcol) * KP + 8 * hh;
+    for (int kk = 0; kk < nkk; ++kk) {
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(ka + 16 * kk));
+      const bf16x8_t bfr = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(qb + 16 * kk));
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr, sc, 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+      const bool valid = rok && j <= jhi && j <= prow && (a.window <= 0 || prow - j < a.window);
+      const float v = valid ? sc[r] * sl2 : -INFINITY;
+      sc[r] = v;
+      mx = fmaxf(mx, v);
+    }
+    mx = xor32_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float alpha = exp2f(m - mn);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float pe = exp2f(sc[r] - mn);
+      sc[r] = pe;
+      sum += pe;
+    }
+    sum = xor32_sum(sum);
+    l = l * alpha + sum;
+    m = mn;
+    bf16x8_t pf[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      uint4 w;
+      w.x = pack2(sc[8 * s2 + 0], sc[8 * s2 + 1]);
+      w.y = pack2(sc[8 * s2 + 2], sc[8 * s2 + 3]);
+      w.z = pack2(sc[8 * s2 + 4], sc[8 * s2 + 5]);
+      w.w = pack2(sc[8 * s2 + 6], sc[8 * s2 + 7]);
+      pf[s2] = __builtin_bit_cast(bf16x8_t, w);
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16x8_t vf = __builtin_bit_cast(
+            bf16x8_t, *reinterpret_cast<const uint4*>(vt + (32 * db + qcol) * VT_PITCH + 16 * s2 + 8 * hh));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[s2], o[db], 0, 0, 0);
+      }
+    }
+  }
+  if (!rok) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  bf16_t* op = reinterpret_cast<bf16_t*>(a.out) + ((int64_t)(myrow % H) * a.total_q + (q0 + myrow / H)) * R;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = 32 * db + 8 * g + 4 * hh;
+      uint2 w;
+      w.x = pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
+      w.y = pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
+      *reinterpret_cast<uint2*>(op + d) = w;
+    }
+  }
+}
+
+inline size_t mfma_lds_bytes(int kp, int ndb) {
+  return sizeof(bf16_t) * ((size_t)(MROWS + MKT) * kp + (size_t)32 * ndb * VT_PITCH);
+}
+
+template <int NDB> hipError_t launch_mfma(const LatentAttnArgs& a, hipStream_t s) {
+  static bool attr_set = false;
+  auto* fn = latent_attn_mfma_kernel<NDB>;
+  const int kp = a.sh.rank + a.sh.rot_dim + 8;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       144 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)(((int64_t)a.max_q * a.heads + MROWS - 1) / MROWS), (unsigned)a.num_seqs);
+  hipLaunchKernelGGL(fn, grid, dim3(256), mfma_lds_bytes(kp, NDB), s, a, kp);
+  return hipGetLastError();
+}
+
+inline bool mfma_ok(const LatentAttnArgs& a) {
+  const int r = a.sh.rank;
+  return !a.f32 && r % 32 == 0 && r <= 256 && a.sh.rot_dim % 16 == 0 && a.q_stride % 1 == 0 &&
+         mfma_lds_bytes(r + a.sh.rot_dim + 8, r / 32) <= 144 * 1024 &&
+         (reinterpret_cast<uintptr_t>(a.q_lat) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.out) & 7) == 0;
+}
+
+hipError_t launch_mfma_any(const LatentAttnArgs& a, hipStream_t s) {
+  switch (a.sh.rank / 32) {
+    case 1: return launch_mfma<1>(a, s);
+    case 2: return launch_mfma<2>(a, s);
+    case 3: return launch_mfma<3>(a, s);
+    case 4: return launch_mfma<4>(a, s);
+    case 5: return launch_mfma<5>(a, s);
+    case 6: return launch_mfma<6>(a, s);
+    case 7: return launch_mfma<7>(a, s);
+    case 8: return launch_mfma<8>(a, s);
+  }
+  return hipErrorInvalidValue;
+}
+
 constexpr int LDS_MAX = 128 * 1024;
 
 inline size_t lds_bytes(int bk, int qs, int ksd) { return sizeof(float) * ((size_t)RW * qs + (size_t)bk * ksd + (size_t)RW * bk); }
@@ -210,6 +419,8 @@ hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s) {
   if (a.heads < 1 || a.sh.rank < 1 || a.sh.rot_dim < 0 || a.sh.rot_pairs * 2 > a.sh.rot_dim || a.block_size < 1 ||
       a.max_q < 1)
     return hipErrorInvalidValue;
+  if (a.impl != 1 && mfma_ok(a)) return launch_mfma_any(a, s);
+  if (a.impl == 2) return hipErrorInvalidValue;  // the matrix-core form was demanded and does not apply
   return a.f32 ? launch_bk<true>(a, s) : launch_bk<false>(a, s);
 }
 

@@ -62,6 +62,7 @@ struct LatentAttnArgs {
   float scale;
   LatentShape sh;
   bool f32;
+  int impl;               // 0: matrix cores where they apply, else the FMA form; 1: FMA form; 2: matrix cores or fail
 };
 hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s);
 

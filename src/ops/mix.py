@@ -155,16 +155,18 @@ def latent_kv_write(cache: torch.Tensor, kv: torch.Tensor, w: torch.Tensor, posi
 def latent_attn(q_lat: torch.Tensor, q: torch.Tensor, rot_off: int, cache: torch.Tensor, block_tables: torch.Tensor,
                 cu_q: Optional[torch.Tensor], ctx_lens: torch.Tensor, positions: torch.Tensor,
                 sink: Optional[torch.Tensor], max_q: int, window: int, scale: float, rot_dim: int,
-                inv_freq: torch.Tensor) -> torch.Tensor:
+                inv_freq: torch.Tensor, impl: int = 0) -> torch.Tensor:
     """Absorbed latent attention. q_lat [H, T, rank]: the queries projected into the latent space; q [T, H * qh]:
     the full queries, head h's rotary part at [h * qh + rot_off, + rot_dim) (rotated here, by positions[t]).
     Row (t, h) scores the cache rows j of its sequence with 0 <= p - j < window (window 0: j <= p):
     (q_lat . latent_j + q_rot . krot_j) * scale, softmax with exp(sink[h]) added to the denominator, and
-    returns the weighted sum of the latent rows, [H, T, rank]. cu_q None: one query row per sequence."""
+    returns the weighted sum of the latent rows, [H, T, rank]. cu_q None: one query row per sequence.
+    ``impl`` (GPU): 0 = the matrix-core kernel where it applies (bf16, rank % 32 == 0, rank <= 256,
+    rot_dim % 16 == 0), else the FMA kernel; 1 = the FMA kernel; 2 = the matrix-core kernel or an error."""
     if not q_lat.is_cuda:
         return ref.latent_attn(q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, window, scale,
                                rot_dim, inv_freq)
     out = torch.empty_like(q_lat)
     _kern().latent_attn(out, q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, max_q, window,
-                        scale, rot_dim, inv_freq)
+                        scale, rot_dim, inv_freq, impl)
     return out

@@ -232,7 +232,8 @@ def _dense_latent_attn(q_lat, q_rot, rows, p, sink, window, scale):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rank,rot,heads,window", [(12, 4, 3, 37), (40, 8, 5, 0), (130, 6, 2, 129), (8, 2, 1, 1)])
+@pytest.mark.parametrize("rank,rot,heads,window", [(12, 4, 3, 37), (40, 8, 5, 0), (130, 6, 2, 129), (8, 2, 1, 1),
+                                                   (64, 16, 6, 37), (96, 0, 2, 0), (256, 32, 7, 129), (32, 16, 1, 16)])
 def test_latent_cache_and_attention_ops(device, dtype, rank, rot, heads, window):
     """latent_kv_write + latent_attn over scattered pages, against a dense computation: one standout key per
     query placed far back, on a page border, just inside and just outside the window (the outside one must be
@@ -277,8 +278,15 @@ def test_latent_cache_and_attention_ops(device, dtype, rank, rot, heads, window)
     bt = perm[None].to(torch.int32).to(device)
     ctx_t = torch.tensor([ctx], dtype=torch.int32, device=device)
     cu = torch.tensor([0, nq], dtype=torch.int32, device=device)
+    # on the GPU in bf16 the shapes the matrix-core kernel takes must really run on it (impl 2 fails otherwise),
+    # and the FMA kernel (impl 1) must agree on the same inputs
+    mfma = device != "cpu" and dtype == torch.bfloat16 and rank % 32 == 0 and rank <= 256 and rot % 16 == 0
     out = ops.latent_attn(q_lat.to(device), q.to(device), 5, cache, bt, cu, ctx_t, p.to(device), sink.to(device), nq,
-                          window, scale, rot, inv)
+                          window, scale, rot, inv, impl=2 if mfma else 0)
+    if mfma:
+        out1 = ops.latent_attn(q_lat.to(device), q.to(device), 5, cache, bt, cu, ctx_t, p.to(device), sink.to(device),
+                               nq, window, scale, rot, inv, impl=1)
+        assert (out.float() - out1.float()).abs().max() < 2e-2 * out1.float().abs().max()
     q_rot = orc.rotate_interleaved(q.view(nq, heads, qh)[:, :, 5:].double(), p, base, rot).transpose(0, 1)
     want = _dense_latent_attn(q_lat.double(), q_rot, rows, p, sink, window, scale)
     tol = 2e-5 if dtype == torch.float32 else 2e-2
