@@ -123,6 +123,10 @@ def parse(argv=None):
     p.add_argument("--node-section-only", action="store_true",
                    help="internal: the node section alone (the child run that rank 0 of a multi-rank run starts)")
     p.add_argument("--verbose", action="store_true")
+    p.add_argument("--design-compare", action="store_true",
+                   help="instead of the serving bench: Datatar beside the closest existing model (Mixtral) at equal "
+                        "sizes, prefill / decode throughput and the attention kernels alone (bench/design_compare.py)")
+    p.add_argument("--design-args", default="", help="arguments passed on to bench/design_compare.py")
     return p.parse_args(argv)
 
 
@@ -454,6 +458,14 @@ class _Watchdog:
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     args = parse(argv)
+    if args.design_compare:  # a separate measurement; the default workload and its JSON contract are untouched
+        import importlib.util
+        import shlex
+
+        spec = importlib.util.spec_from_file_location("design_compare", os.path.join(ROOT, "bench", "design_compare.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod.main(shlex.split(args.design_args))
     if needs_launcher(args):
         return self_launch(args, argv)
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -216,6 +216,32 @@ void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cac
   a.sh = latent_shape(rank, rot_dim, inv_freq);
   a.f32 = f;
   a.impl = (int)impl;
+  a.ws_o = a.ws_ml = nullptr;
+  a.nsplit = 1;
+  a.chunk = 0;
+  Tensor ws_o, ws_ml;
+  if (die::latent_attn_uses_mfma(a)) {
+    // few row tiles (decode steps): split the keys over workgroups until about 256 are in flight. The key range
+    // is bounded by the window, else by the block table's width (under a captured graph: the model length;
+    // splits beyond a sequence's keys exit at once)
+    const int64_t rows_wg = max_q * H <= 32 ? 32 : 128;
+    const int64_t tiles = S * ((max_q * H + rows_wg - 1) / rows_wg);
+    int64_t bound = block_tables.size(1) * cache.size(1);
+    if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
+    int64_t ns = std::min<int64_t>({(int64_t)16, 256 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
+    if (ns > 1) {
+      a.chunk = (int)((((bound + ns - 1) / ns) + 31) / 32 * 32);
+      a.nsplit = (int)((bound + a.chunk - 1) / a.chunk);
+      if (a.nsplit > 1) {
+        ws_o = at::empty({a.nsplit, H * T, rank}, q_lat.options().dtype(at::kFloat));
+        ws_ml = at::empty({a.nsplit, H * T, 2}, q_lat.options().dtype(at::kFloat));
+        a.ws_o = ws_o.data_ptr<float>();
+        a.ws_ml = ws_ml.data_ptr<float>();
+      } else {
+        a.nsplit = 1;
+      }
+    }
+  }
   HIP_OK(die::launch_latent_attn(a, cur_stream()));
 }
 

@@ -167,40 +167,61 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(LatentAttnArgs a, int 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// bf16 on the matrix cores (v_mfma_f32_32x32x16_bf16), for rank % 32 == 0, rank <= 256, rot_dim % 16 == 0.
-// Workgroup = 4 waves x 32 rows. Per tile of 32 keys, staged once in LDS both row-major (K: [key][Dk]) and
-// transposed (V^T: [d][key'], key' = the key order of the score accumulator's rows, so a PV operand is one
-// 16-byte read):
+// bf16 on the matrix cores (v_mfma_f32_32x32x16_bf16), for rank % 32 == 0, rank <= 256, rot_dim % 16 == 0,
+// rot_dim <= 128. Workgroup = NW waves x 32 rows (NW = 1 for steps of few rows per sequence: decode). Per
+// tile of 32 keys, staged once in LDS row-major ([key][Dk], the next tile's global loads in flight meanwhile):
 //   S^T[key][q] = K Q^T        A = K rows from LDS, B = Q rows from LDS      (Dk / 16 MFMAs)
 //   online softmax per query column (one lane pair owns a query: no cross-lane traffic beyond xor 32),
 //   fp32 scores and weights, running max seeded with the sink; P is rounded to bf16 only as the MFMA operand
-//   O^T[d][q] += V^T P^T      A = V^T from LDS, B = P^T from the accumulator  (2 * rank / 32 MFMAs)
-constexpr int MROWS = 128, MKT = 32, VT_PITCH = 40;  // V^T row pitch in bf16 (80 B: 16-byte aligned reads)
+//   O^T[d][q] += V^T P^T      A = the latent columns of the same tile, read transposed (ds_read_tr16_b64),
+//                              B = P^T straight from the score accumulator  (2 * rank / 32 MFMAs)
+// Split keys (grid.z = nsplit > 1; decode over long contexts): split z takes keys [jlo + z * chunk, + chunk),
+// writes its unnormalised O, running max and sum to a workspace, and latent_attn_merge_kernel combines them;
+// the sink enters split 0 only.
+constexpr int MKT = 32;
+typedef __attribute__((address_space(3))) short4_t lds_short4;
+typedef __attribute__((ext_vector_type(8))) short short8_t;
 
-template <int NDB>
-__global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a, int KP) {
+template <int NDB, int NW>
+__global__ void __launch_bounds__(64 * NW) latent_attn_mfma_kernel(LatentAttnArgs a, int KP) {
+  constexpr int ROWS = 32 * NW, NT = 64 * NW;
+  constexpr int NPF = (MKT * (4 * NDB + 16) + NT - 1) / NT;  // 16-byte chunks of a key tile per thread (rot_dim <= 128)
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [MROWS][KP]
-  bf16_t* ks = qs + MROWS * KP;                               // [MKT][KP]
-  bf16_t* vt = ks + MKT * KP;                                 // [32 * NDB][VT_PITCH]
-  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [ROWS][KP]
+  bf16_t* ks = qs + ROWS * KP;                                // [MKT][KP]
+  const int s = blockIdx.y, z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
   const int H = a.heads, R = a.sh.rank, Dk = a.sh.rank + a.sh.rot_dim;
   const int q0 = a.cu_q ? a.cu_q[s] : s;
   const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
-  const int nrows = nq * H, row0 = blockIdx.x * MROWS;
+  const int nrows = nq * H, row0 = blockIdx.x * ROWS;
   if (row0 >= nrows) return;
   const int ctx = a.ctx_lens[s];
-  const int last_row = min(row0 + MROWS, nrows) - 1;
+  const int last_row = min(row0 + ROWS, nrows) - 1;
   const int p_first = (int)a.positions[q0 + row0 / H], p_last = (int)a.positions[q0 + last_row / H];
-  const int jlo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
-  const int jhi = min(p_last, ctx - 1);
+  int jlo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  int jhi = min(p_last, ctx - 1);
+  if (a.nsplit > 1) {
+    jlo += z * a.chunk;
+    jhi = min(jhi, jlo + a.chunk - 1);
+  }
   const bf16_t* qlat = reinterpret_cast<const bf16_t*>(a.q_lat);
   const bf16_t* qrot = reinterpret_cast<const bf16_t*>(a.q_rot);
   const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+  const int qcol = lane & 31, hh = lane >> 5;
+  const int myrow = row0 + wave * 32 + qcol;
+  const bool rok = myrow < nrows;
+  const int64_t orow = rok ? (int64_t)(myrow % H) * a.total_q + (q0 + myrow / H) : 0;
+  if (jlo > jhi) {  // an empty split (uniform over the workgroup): it only reports that it holds nothing
+    if (a.nsplit > 1 && rok && hh == 0) {
+      a.ws_ml[((int64_t)z * a.heads * a.total_q + orow) * 2] = -1e30f;
+      a.ws_ml[((int64_t)z * a.heads * a.total_q + orow) * 2 + 1] = 0.f;
+    }
+    return;
+  }
 
   // queries -> LDS: the latent part as 16-byte copies, the rotary part rotated in fp32
   const int lch = R / 8;
-  for (int idx = tid; idx < MROWS * lch; idx += 256) {
+  for (int idx = tid; idx < ROWS * lch; idx += NT) {
     const int r = idx / lch, c = idx % lch, row = row0 + r;
     uint4 v = make_uint4(0, 0, 0, 0);
     if (row < nrows) {
@@ -209,7 +230,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a,
     }
     *reinterpret_cast<uint4*>(qs + r * KP + 8 * c) = v;
   }
-  for (int idx = tid; idx < MROWS * a.sh.rot_dim; idx += 256) {
+  for (int idx = tid; idx < ROWS * a.sh.rot_dim; idx += NT) {
     const int r = idx / a.sh.rot_dim, dd = idx % a.sh.rot_dim, row = row0 + r;
     float v = 0.f;
     if (row < nrows) {
@@ -228,14 +249,11 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a,
     qs[r * KP + R + dd] = f2bf(v);
   }
 
-  const int qcol = lane & 31, hh = lane >> 5;
-  const int myrow = row0 + wave * 32 + qcol;
-  const bool rok = myrow < nrows;
   const bool wave_live = row0 + wave * 32 < nrows;
   const int prow = rok ? (int)a.positions[q0 + myrow / H] : -1;
   constexpr float LOG2E = 1.4426950408889634f;
   const float sl2 = a.scale * LOG2E;
-  const bool has_sink = a.sink != nullptr && rok;
+  const bool has_sink = a.sink != nullptr && rok && z == 0;
   float m = has_sink ? a.sink[myrow % H] * LOG2E : -1e30f;
   float l = has_sink ? 1.0f : 0.0f;
   f32x16_t o[NDB];
@@ -245,24 +263,33 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a,
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
 
   const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
-  const int kch = Dk / 8, nkk = Dk / 16;
-  for (int j0 = jlo; j0 <= jhi; j0 += MKT) {
-    __syncthreads();
-    for (int idx = tid; idx < MKT * kch; idx += 256) {
-      const int k = idx / kch, c = idx % kch, j = j0 + k;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (j <= jhi) v = *reinterpret_cast<const uint4*>(
-          cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
-      *reinterpret_cast<uint4*>(ks + k * KP + 8 * c) = v;
-      if (8 * c < R) {
-        const int k16 = k & 15;
-        const int kp = (k & 16) + 8 * ((k16 >> 2) & 1) + (k16 & 3) + 4 * (k16 >> 3);
-        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+  const int kch = Dk / 8, nkk = Dk / 16, nchunks = MKT * kch;
+  uint4 pf[NPF];
+  auto fetch = [&](int j0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vt[(8 * c + e) * VT_PITCH + kp] = (bf16_t)((wv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-      }
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      const int k = idx / kch, c = idx % kch, j = j0 + k;
+      pf[u] = make_uint4(0, 0, 0, 0);
+      if (idx < nchunks && j <= jhi)
+        pf[u] = *reinterpret_cast<const uint4*>(
+            cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
+    }
+  };
+  fetch(jlo);
+  const int pitchB = KP * 2;
+  const int g16 = lane >> 4, i16 = lane & 15;
+  const char* vbase = reinterpret_cast<const char*>(ks) + (4 * hh + (i16 >> 2)) * pitchB +
+                      (16 * (g16 & 1) + 4 * (i16 & 3)) * 2;
+  for (int j0 = jlo; j0 <= jhi; j0 += MKT) {
+    __syncthreads();  // every wave is done with the previous tile (first: the queries are being written)
+#pragma unroll
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      if (idx < nchunks) *reinterpret_cast<uint4*>(ks + (idx / kch) * KP + 8 * (idx % kch)) = pf[u];
     }
     __syncthreads();
+    if (j0 + MKT <= jhi) fetch(j0 + MKT);  // in flight while this tile is computed
     if (!wave_live) continue;
     f32x16_t sc;
 #pragma unroll
@@ -296,7 +323,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a,
     sum = xor32_sum(sum);
     l = l * alpha + sum;
     m = mn;
-    bf16x8_t pf[2];
+    bf16x8_t pfr[2];
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
       uint4 w;
@@ -304,43 +331,80 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatentAttnArgs a,
       w.y = pack2(sc[8 * s2 + 2], sc[8 * s2 + 3]);
       w.z = pack2(sc[8 * s2 + 4], sc[8 * s2 + 5]);
       w.w = pack2(sc[8 * s2 + 6], sc[8 * s2 + 7]);
-      pf[s2] = __builtin_bit_cast(bf16x8_t, w);
+      pfr[s2] = __builtin_bit_cast(bf16x8_t, w);
     }
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
+      if (alpha != 1.0f) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const bf16x8_t vf = __builtin_bit_cast(
-            bf16x8_t, *reinterpret_cast<const uint4*>(vt + (32 * db + qcol) * VT_PITCH + 16 * s2 + 8 * hh));
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[s2], o[db], 0, 0, 0);
+        const char* a0 = vbase + (16 * s2) * pitchB + 64 * db;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0 + 8 * pitchB));
+        const short8_t a8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a8), pfr[s2], o[db], 0, 0, 0);
       }
     }
   }
   if (!rok) return;
+  if (a.nsplit > 1) {
+    float* wo = a.ws_o + ((int64_t)z * a.heads * a.total_q + orow) * R;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<float4*>(wo + 32 * db + 8 * g + 4 * hh) =
+            make_float4(o[db][4 * g], o[db][4 * g + 1], o[db][4 * g + 2], o[db][4 * g + 3]);
+    if (hh == 0) {
+      a.ws_ml[((int64_t)z * a.heads * a.total_q + orow) * 2] = m;
+      a.ws_ml[((int64_t)z * a.heads * a.total_q + orow) * 2 + 1] = l;
+    }
+    return;
+  }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
-  bf16_t* op = reinterpret_cast<bf16_t*>(a.out) + ((int64_t)(myrow % H) * a.total_q + (q0 + myrow / H)) * R;
+  bf16_t* op = reinterpret_cast<bf16_t*>(a.out) + orow * R;
 #pragma unroll
   for (int db = 0; db < NDB; ++db) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const int d = 32 * db + 8 * g + 4 * hh;
       uint2 w;
       w.x = pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
       w.y = pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-      *reinterpret_cast<uint2*>(op + d) = w;
+      *reinterpret_cast<uint2*>(op + 32 * db + 8 * g + 4 * hh) = w;
     }
   }
 }
 
-inline size_t mfma_lds_bytes(int kp, int ndb) {
-  return sizeof(bf16_t) * ((size_t)(MROWS + MKT) * kp + (size_t)32 * ndb * VT_PITCH);
+// out[row] = sum_z O_z 2^(m_z - m*) / sum_z l_z 2^(m_z - m*), m* = max_z m_z (running maxima in log2 units).
+__global__ void __launch_bounds__(256) latent_attn_merge_kernel(bf16_t* out, const float* ws_o, const float* ws_ml,
+                                                                int nsplit, int64_t rows, int R) {
+  const int64_t row = blockIdx.x;
+  float mstar = -1e30f;
+  for (int z = 0; z < nsplit; ++z) mstar = fmaxf(mstar, ws_ml[((int64_t)z * rows + row) * 2]);
+  float lsum = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
+    if (lz > 0.f) lsum += lz * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
+  }
+  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  for (int c = threadIdx.x; c < R; c += 256) {
+    float acc = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
+      if (lz > 0.f) acc += ws_o[((int64_t)z * rows + row) * R + c] * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
+    }
+    out[row * R + c] = f2bf(acc * inv);
+  }
 }
 
-template <int NDB> hipError_t launch_mfma(const LatentAttnArgs& a, hipStream_t s) {
+inline size_t mfma_lds_bytes(int kp, int nw) { return sizeof(bf16_t) * (size_t)(32 * nw + MKT) * kp; }
+
+template <int NDB, int NW> hipError_t launch_mfma(const LatentAttnArgs& a, hipStream_t s) {
   static bool attr_set = false;
-  auto* fn = latent_attn_mfma_kernel<NDB>;
+  auto* fn = latent_attn_mfma_kernel<NDB, NW>;
   const int kp = a.sh.rank + a.sh.rot_dim + 8;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -348,31 +412,41 @@ template <int NDB> hipError_t launch_mfma(const LatentAttnArgs& a, hipStream_t s
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const dim3 grid((unsigned)(((int64_t)a.max_q * a.heads + MROWS - 1) / MROWS), (unsigned)a.num_seqs);
-  hipLaunchKernelGGL(fn, grid, dim3(256), mfma_lds_bytes(kp, NDB), s, a, kp);
+  const dim3 grid((unsigned)(((int64_t)a.max_q * a.heads + 32 * NW - 1) / (32 * NW)), (unsigned)a.num_seqs,
+                  (unsigned)max(1, a.nsplit));
+  hipLaunchKernelGGL(fn, grid, dim3(64 * NW), mfma_lds_bytes(kp, NW), s, a, kp);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || a.nsplit <= 1) return e;
+  hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)((int64_t)a.heads * a.total_q)), dim3(256), 0, s,
+                     reinterpret_cast<bf16_t*>(a.out), a.ws_o, a.ws_ml, a.nsplit, (int64_t)a.heads * a.total_q,
+                     a.sh.rank);
   return hipGetLastError();
 }
 
 inline bool mfma_ok(const LatentAttnArgs& a) {
   const int r = a.sh.rank;
-  return !a.f32 && r % 32 == 0 && r <= 256 && a.sh.rot_dim % 16 == 0 && a.q_stride % 1 == 0 &&
-         mfma_lds_bytes(r + a.sh.rot_dim + 8, r / 32) <= 144 * 1024 &&
+  return !a.f32 && r % 32 == 0 && r <= 256 && a.sh.rot_dim % 16 == 0 && a.sh.rot_dim <= 128 &&
          (reinterpret_cast<uintptr_t>(a.q_lat) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0 &&
          (reinterpret_cast<uintptr_t>(a.out) & 7) == 0;
 }
 
-hipError_t launch_mfma_any(const LatentAttnArgs& a, hipStream_t s) {
+template <int NW> hipError_t launch_mfma_ndb(const LatentAttnArgs& a, hipStream_t s) {
   switch (a.sh.rank / 32) {
-    case 1: return launch_mfma<1>(a, s);
-    case 2: return launch_mfma<2>(a, s);
-    case 3: return launch_mfma<3>(a, s);
-    case 4: return launch_mfma<4>(a, s);
-    case 5: return launch_mfma<5>(a, s);
-    case 6: return launch_mfma<6>(a, s);
-    case 7: return launch_mfma<7>(a, s);
-    case 8: return launch_mfma<8>(a, s);
+    case 1: return launch_mfma<1, NW>(a, s);
+    case 2: return launch_mfma<2, NW>(a, s);
+    case 3: return launch_mfma<3, NW>(a, s);
+    case 4: return launch_mfma<4, NW>(a, s);
+    case 5: return launch_mfma<5, NW>(a, s);
+    case 6: return launch_mfma<6, NW>(a, s);
+    case 7: return launch_mfma<7, NW>(a, s);
+    case 8: return launch_mfma<8, NW>(a, s);
   }
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_mfma_any(const LatentAttnArgs& a, hipStream_t s) {
+  // one wave per workgroup when a sequence brings at most 32 rows (decode steps): small LDS, many workgroups
+  return (int64_t)a.max_q * a.heads <= 32 ? launch_mfma_ndb<1>(a, s) : launch_mfma_ndb<4>(a, s);
 }
 
 constexpr int LDS_MAX = 128 * 1024;
@@ -413,6 +487,8 @@ template <bool F32> hipError_t launch_bk(const LatentAttnArgs& a, hipStream_t s)
 }
 
 }  // namespace
+
+bool latent_attn_uses_mfma(const LatentAttnArgs& a) { return a.impl != 1 && mfma_ok(a); }
 
 hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s) {
   if (a.num_seqs == 0 || a.total_q == 0) return hipSuccess;

@@ -62,8 +62,17 @@ struct LatentAttnArgs {
   float scale;
   LatentShape sh;
   bool f32;
+  // split keys (matrix-core kernel only): nsplit > 1 workgroups per row tile take `chunk` keys each and write
+  // unnormalised partial sums to ws_o [nsplit, H * T, rank] and (running max in log2 units, sum) to
+  // ws_ml [nsplit, H * T, 2]; a merge kernel then writes `out`
+  float* ws_o;
+  float* ws_ml;
+  int nsplit, chunk;
   int impl;               // 0: matrix cores where they apply, else the FMA form; 1: FMA form; 2: matrix cores or fail
 };
 hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s);
+// whether launch_latent_attn would run the matrix-core kernel for these arguments (the split workspace is only
+// used by it)
+bool latent_attn_uses_mfma(const LatentAttnArgs& a);
 
 }  // namespace die

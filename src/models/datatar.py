@@ -246,8 +246,8 @@ class LatentAttentionMixer:
     def forward(self, a: torch.Tensor, positions: torch.Tensor, meta, cache: torch.Tensor, eps: float) -> torch.Tensor:
         s = self.spec
         t = a.shape[0]
-        p = F.linear(a, self.dqkv)
-        q = F.linear(mix.rms_norm_ext(p[:, : s.q_rank], self.dq_norm, eps), self.uq)
+        p = mix.linear(a, self.dqkv)
+        q = mix.linear(mix.rms_norm_ext(p[:, : s.q_rank], self.dq_norm, eps), self.uq)
         mix.latent_kv_write(cache, p[:, s.q_rank:], self.dkv_norm, positions, meta.slot_mapping, s.kv_rank, s.rot_dim,
                             self.inv_freq, eps)
         q_lat = torch.bmm(q.view(t, s.heads, s.dim + s.rot_dim)[:, :, : s.dim].transpose(0, 1), self.uk)
@@ -255,7 +255,7 @@ class LatentAttentionMixer:
                                 meta.ctx_lens, positions, self.sink, meta.max_q_len if meta.is_prefill else 1,
                                 s.window, s.scale, s.rot_dim, self.inv_freq)
         o = torch.bmm(o_lat, self.uv_t).transpose(0, 1).reshape(t, s.heads * s.vdim)
-        return F.linear(o, self.o)
+        return mix.linear(o, self.o)
 
 
 MIXERS = {LatentAttentionMixer.type_name: LatentAttentionMixer}
@@ -496,15 +496,15 @@ class DatatarLM:
 
     def _mlp(self, lw: MixLayerWeights, f: MlpSpec, a: torch.Tensor) -> torch.Tensor:
         if f.kind == "dense":
-            return F.linear(mix.gated_act(F.linear(a, lw.gate_up), mix.ACT_CLAMPED, f.limit, GATE_ALPHA), lw.down)
+            return mix.linear(mix.gated_act(mix.linear(a, lw.gate_up), mix.ACT_CLAMPED, f.limit, GATE_ALPHA), lw.down)
         w, ids = mix.route_sigmoid_topk(a, lw.router, f.top)
         shared = None
         if lw.shared_gate_up is not None:
-            shared = F.linear(mix.gated_act(F.linear(a, lw.shared_gate_up), mix.ACT_SILU), lw.shared_down)
+            shared = mix.linear(mix.gated_act(mix.linear(a, lw.shared_gate_up), mix.ACT_SILU), lw.shared_down)
         return mix.moe_input_scaled(a, lw.w13, lw.w2, w, ids, extra=shared)
 
     def compute_logits(self, hidden: torch.Tensor, argmax_parts=None) -> torch.Tensor:
         """fp32 logits [rows, vocab] = head(hidden) * logit_scale."""
         if argmax_parts is not None:
             raise ValueError("this head writes no per-tile argmax candidates")
-        return F.linear(hidden, self.lm_head).float() * self.arch.logit_scale
+        return mix.linear(hidden, self.lm_head).float() * self.arch.logit_scale

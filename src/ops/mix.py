@@ -93,6 +93,18 @@ def route_sigmoid_topk(x: torch.Tensor, router: torch.Tensor, k: int) -> Tuple[t
     return w, ids
 
 
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """y = x @ w^T. bf16 steps of up to 128 rows go through :func:`src.ops.linear` (the weight-streaming decode
+    GEMM where the shape tiles it) when the Llama-path extension is loaded; everything else is the library GEMM
+    (fp32 inputs: true fp32)."""
+    if x.is_cuda and x.dtype == torch.bfloat16 and 0 < x.shape[0] <= 128 and x.is_contiguous():
+        from src import ops
+
+        if ops.native_available():
+            return ops.linear(x, w)
+    return F.linear(x, w)
+
+
 # (token, expert) rows up to which the experts' weights are gathered per row for two batched GEMMs (no host
 # read, hipGraph-capturable: decode steps); above it each expert runs one library GEMM pair over its rows
 MOE_BMM_MAX_ROWS = 64
@@ -113,6 +125,27 @@ def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: to
     w = w.contiguous()
     out = torch.empty(t, h, dtype=torch.float32, device=x.device)
     xs = torch.empty(n, h, dtype=x.dtype, device=x.device)
+    if x.dtype == torch.bfloat16 and t <= 128:
+        # decode-sized steps: the framework's expert-streaming grouped GEMM (every routed expert's weights
+        # streamed once, SiLU * up fused; no host read, hipGraph-capturable) on the scaled, expert-sorted rows
+        from src import ops
+
+        tiles = ops._moe_decode_tiles(h, w13.shape[1] // 2, t) if ops.native_available() else None
+        if tiles is not None:
+            ck = ops._kern()
+            (wr1, kc1), (wr2, kc2) = tiles
+            offsets = torch.empty(e + 1, dtype=torch.int32, device=x.device)
+            sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
+            pos = torch.empty(n, dtype=torch.int32, device=x.device)
+            kern.moe_align(offsets, sorted_idx, pos, ids.reshape(-1).contiguous(), e)
+            kern.gather_scaled(xs, x, sorted_idx, w, k)
+            a = torch.empty(n, w13.shape[1] // 2, dtype=x.dtype, device=x.device)
+            ys = torch.empty(n, h, dtype=x.dtype, device=x.device)
+            none = ops._NO_ROWS(x.device)
+            ck.gemm_decode_grouped(a, xs, w13, offsets, 1, wr1, kc1, none, 1, t, 1)
+            ck.gemm_decode_grouped(ys, a, w2, offsets, 0, wr2, kc2, none, 1, t, 1)
+            kern.combine_sum(out, ys, pos, extra, k)
+            return out
     if n <= MOE_BMM_MAX_ROWS or torch.cuda.is_current_stream_capturing():
         kern.gather_scaled(xs, x, None, w, k)
         sel = ids.reshape(-1).long()

@@ -538,3 +538,35 @@ def test_trace_runner_command_line(tmp_path):
     assert rel_err(b, orc.forward(wts, cfg, toks[:3])[[2]]) < TOL[torch.float32]
     c = torch.from_numpy(np.fromfile(tmp_path / "o" / "2.f32", dtype="<f4").reshape(1, -1))
     assert rel_err(c, want[[39]]) < TOL[torch.float32]
+
+
+@pytest.mark.gpu
+def test_generation_with_decode_graphs_and_decode_gemms(tmp_path):
+    """Served configuration: shapes that the weight-streaming decode GEMM and the expert-streaming grouped GEMM
+    tile (width 256, expert width 64), the matrix-core attention (rank 64, rot 16), decode steps replayed from
+    captured hipGraphs in multi-step windows. Every replay's token is checked against the oracle."""
+    _need("cuda:0")
+    from src.preproc import SamplingParams
+
+    mixer = orc.mixer_cfg(heads=4, dim=48, rot_dim=16, vdim=32, kv_rank=64, q_rank=96, window=24)
+    cfg = orc.make_config([(mixer, orc.dense_cfg(ff=256)), (mixer, orc.moe_cfg(experts=4, top=2, ff=64, shared=64))],
+                          vocab=128, width=256)
+    wts = orc.make_weights(cfg, seed=21)
+    eng = make_engine(tmp_path, cfg, wts, "cuda:0", torch.bfloat16, max_tokens=1024, max_seqs=4, use_cuda_graph=True,
+                      graph_batch_sizes=[1, 2, 4], decode_window=4)
+    eng.eos_token_id = None
+    eng.runner.capture_graphs()
+    assert eng.runner.graph_sizes == [1, 2, 4]
+    prompts = [tokens_for(cfg, n, 30 + n) for n in (7, 33, 20)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=40))
+    assert [len(o) for o in outs] == [40, 40, 40]
+    assert eng.stats.get("decode_windows", 0) >= 5
+    for p, o in zip(prompts, outs):
+        lg = orc.forward(wts, cfg, p + o)
+        for i, tok in enumerate(o):
+            row = lg[len(p) + i - 1]
+            assert float(row.max() - row[tok]) <= 0.05 * float(row.max() - row.min()), (i, tok, int(row.argmax()))
+    # the same prompts teacher-forced through replay_step (eager, no graphs) give the oracle's logits
+    got = replay(eng, cut("z", prompts[1] + outs[1], [len(prompts[1])]))["z"]
+    check_against_oracle(got, wts, cfg, prompts[1] + outs[1], TOL[torch.bfloat16])
+    assert eng.blocks.num_available() == eng.blocks.num_blocks
