@@ -178,6 +178,8 @@ def main(argv=None) -> int:
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--window", type=int, default=0, help="Datatar's sliding window (0: full context, as the GQA path)")
     ap.add_argument("--skip-serving", action="store_true")
+    ap.add_argument("--skip-kernels", action="store_true")
+    ap.add_argument("--models", default="datatar,mixtral", help="which models to serve")
     a = ap.parse_args(argv)
     assert torch.cuda.is_available(), "needs a GPU"
     from src.models.datatar import DatatarLM
@@ -187,11 +189,15 @@ def main(argv=None) -> int:
     summary = []
     for size in a.sizes.split(","):
         z = SIZES[size]
-        summary += attention_kernels(z, a, size)
+        if not a.skip_kernels:
+            summary += attention_kernels(z, a, size)
         if a.skip_serving:
             continue
-        summary.append(serve(DatatarLM(datatar_arch(z, a.window), "cuda:0", seed=1, init_std=0.02), a, "datatar", size))
-        summary.append(serve(CausalLM(mixtral_arch(z), "cuda:0", seed=1), a, "mixtral", size))
+        if "datatar" in a.models.split(","):
+            summary.append(serve(DatatarLM(datatar_arch(z, a.window), "cuda:0", seed=1, init_std=0.02), a, "datatar",
+                                 size))
+        if "mixtral" in a.models.split(","):
+            summary.append(serve(CausalLM(mixtral_arch(z), "cuda:0", seed=1), a, "mixtral", size))
     print(json.dumps({"bench": "design_compare_summary", "seconds": round(time.time() - t0, 1), "rows": summary}),
           flush=True)
     return 0

@@ -94,6 +94,17 @@ void route_sigmoid_topk(Tensor w, Tensor ids, Tensor x, Tensor wr) {
                                         (int)w.size(1), cur_stream()));
 }
 
+void topk_sigmoid(Tensor w, Tensor ids, Tensor z) {
+  check_i(w, at::kFloat, "w");
+  check_i(ids, at::kInt, "ids");
+  check_i(z, at::kFloat, "z");
+  TORCH_CHECK(z.dim() == 2 && w.dim() == 2 && w.size(0) == z.size(0) && ids.sizes() == w.sizes() &&
+                  w.size(1) <= z.size(1),
+              "z [T, E]; w, ids [T, K], K <= E");
+  HIP_OK(die::launch_topk_sigmoid(w.data_ptr<float>(), ids.data_ptr<int>(), z.data_ptr<float>(), (int)z.size(0),
+                                  (int)z.size(1), (int)w.size(1), cur_stream()));
+}
+
 void gather_scaled(Tensor xs, Tensor x, OptTensor sorted, Tensor w, int64_t topk) {
   const bool f = is_f32(x, "x");
   check_i(w, at::kFloat, "w");
@@ -228,7 +239,7 @@ void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cac
     const int64_t tiles = S * ((max_q * H + rows_wg - 1) / rows_wg);
     int64_t bound = block_tables.size(1) * cache.size(1);
     if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
-    int64_t ns = std::min<int64_t>({(int64_t)16, 256 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
+    int64_t ns = std::min<int64_t>({(int64_t)16, 512 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
     if (ns > 1) {
       a.chunk = (int)((((bound + ns - 1) / ns) + 31) / 32 * 32);
       a.nsplit = (int)((bound + a.chunk - 1) / a.chunk);
@@ -263,6 +274,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("post_norm_residual", &post_norm_residual);
   m.def("gated_act", &gated_act);
   m.def("route_sigmoid_topk", &route_sigmoid_topk);
+  m.def("topk_sigmoid", &topk_sigmoid);
   m.def("gather_scaled", &gather_scaled);
   m.def("combine_sum", &combine_sum);
   m.def("latent_kv_write", &latent_kv_write);

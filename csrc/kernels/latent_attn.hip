@@ -444,7 +444,250 @@ template <int NW> hipError_t launch_mfma_ndb(const LatentAttnArgs& a, hipStream_
   return hipErrorInvalidValue;
 }
 
+// Prompt-sized steps at the common rotary widths (rot_dim = 16 * NROT): the same algorithm with every wave's
+// query fragments held in registers (loaded straight from global memory, the rotary part rotated on the way;
+// no query tile in LDS, so the per-tile LDS traffic is the key tile alone) and the key tile double-buffered
+// (one barrier per tile: the next tile's registers are stored into the other buffer after this tile's MFMAs).
+template <int NDB, int NROT>
+__global__ void __launch_bounds__(256) latent_attn_mfma_rq_kernel(LatentAttnArgs a, int KP) {
+  constexpr int NT = 256, NKK = 2 * NDB + NROT, KCH = 4 * NDB + 2 * NROT, NCH = MKT * KCH;
+  constexpr int NPF = (NCH + NT - 1) / NT;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  bf16_t* ks0 = reinterpret_cast<bf16_t*>(smem_raw);          // 2 x [MKT][KP]
+  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  const int H = a.heads;
+  constexpr int R = 32 * NDB, Dk = R + 16 * NROT;
+  const int q0 = a.cu_q ? a.cu_q[s] : s;
+  const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
+  const int nrows = nq * H, row0 = blockIdx.x * 128;
+  if (row0 >= nrows) return;
+  const int ctx = a.ctx_lens[s];
+  const int last_row = min(row0 + 128, nrows) - 1;
+  const int p_first = (int)a.positions[q0 + row0 / H], p_last = (int)a.positions[q0 + last_row / H];
+  const int jlo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  const int jhi = min(p_last, ctx - 1);
+  const bf16_t* qlat = reinterpret_cast<const bf16_t*>(a.q_lat);
+  const bf16_t* qrot = reinterpret_cast<const bf16_t*>(a.q_rot);
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+  const int qcol = lane & 31, hh = lane >> 5;
+  const int myrow = row0 + wave * 32 + qcol;
+  const bool rok = myrow < nrows;
+  const bool wave_live = row0 + wave * 32 < nrows;
+  const int64_t tq = rok ? q0 + myrow / H : 0;
+  const int hq = rok ? myrow % H : 0;
+  const int64_t orow = (int64_t)hq * a.total_q + tq;
+  const int prow = rok ? (int)a.positions[tq] : -1;
+  const int wrow_lo = row0 + wave * 32;
+  const bool all_rows = wrow_lo + 31 < nrows;
+  const int pw_min = wave_live ? (int)a.positions[q0 + wrow_lo / H] : 0;
+  const int pw_max = wave_live ? (int)a.positions[q0 + min(wrow_lo + 31, nrows - 1) / H] : 0;
+
+  // this lane's query fragments: qf[kk] = Q[row][16 kk + 8 hh .. + 8]
+  bf16x8_t qf[NKK];
+#pragma unroll
+  for (int kk = 0; kk < 2 * NDB; ++kk) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (rok) v = *reinterpret_cast<const uint4*>(qlat + orow * R + 16 * kk + 8 * hh);
+    qf[kk] = __builtin_bit_cast(bf16x8_t, v);
+  }
+#pragma unroll
+  for (int kr = 0; kr < NROT; ++kr) {
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = 0.f;
+    if (rok) {
+      const bf16_t* qp = qrot + tq * a.q_stride + (int64_t)hq * a.q_hstride + 16 * kr + 8 * hh;
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        const int i = (16 * kr + 8 * hh) / 2 + pr;
+        const float u = bf2f(qp[2 * pr]), w = bf2f(qp[2 * pr + 1]);
+        if (i < a.sh.rot_pairs) {
+          float sn, cs;
+          sincosf((float)prow * a.sh.inv_freq[i], &sn, &cs);
+          f[2 * pr] = u * cs - w * sn;
+          f[2 * pr + 1] = w * cs + u * sn;
+        } else {
+          f[2 * pr] = u;
+          f[2 * pr + 1] = w;
+        }
+      }
+    }
+    qf[2 * NDB + kr] = __builtin_bit_cast(bf16x8_t, pack8(f));
+  }
+
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float sl2 = a.scale * LOG2E;
+  const bool has_sink = a.sink != nullptr && rok;
+  float m = has_sink ? a.sink[hq] * LOG2E : -1e30f;
+  float l = has_sink ? 1.0f : 0.0f;
+  f32x16_t o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+
+  const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
+  uint4 pf[NPF];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      const int k = idx / KCH, c = idx % KCH, j = j0 + k;
+      pf[u] = make_uint4(0, 0, 0, 0);
+      if (idx < NCH && j <= jhi)
+        pf[u] = *reinterpret_cast<const uint4*>(
+            cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
+    }
+  };
+  auto stash = [&](bf16_t* ks) {
+#pragma unroll
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      if (idx < NCH) *reinterpret_cast<uint4*>(ks + (idx / KCH) * KP + 8 * (idx % KCH)) = pf[u];
+    }
+  };
+  fetch(jlo);
+  stash(ks0);
+  if (jlo + MKT <= jhi) fetch(jlo + MKT);
+  const int pitchB = KP * 2;
+  const int g16 = lane >> 4, i16 = lane & 15;
+  const int voff = (4 * hh + (i16 >> 2)) * pitchB + (16 * (g16 & 1) + 4 * (i16 & 3)) * 2;
+  int cur = 0;
+  for (int j0 = jlo; j0 <= jhi; j0 += MKT, cur ^= 1) {
+    __syncthreads();  // tile j0 is complete in buffer cur; every wave has left the other buffer
+    bf16_t* ks = ks0 + cur * (MKT * KP);
+    if (wave_live) {
+      f32x16_t sc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+      const bf16_t* ka = ks + qcol * KP + 8 * hh;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(ka + 16 * kk));
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, qf[kk], sc, 0, 0, 0);
+      }
+      float mx = -INFINITY;
+      // interior tiles (every key visible to every row of the wave) skip the per-score mask
+      if (all_rows && j0 + MKT - 1 <= min(pw_min, jhi) && (a.window <= 0 || pw_max - j0 < a.window)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sc[r] *= sl2;
+          mx = fmaxf(mx, sc[r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+          const bool valid = rok && j <= jhi && j <= prow && (a.window <= 0 || prow - j < a.window);
+          const float v = valid ? sc[r] * sl2 : -INFINITY;
+          sc[r] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+      mx = xor32_max(mx);
+      const float mn = fmaxf(m, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m - mn);
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pe = __builtin_amdgcn_exp2f(sc[r] - mn);
+        sc[r] = pe;
+        sum += pe;
+      }
+      sum = xor32_sum(sum);
+      l = l * alpha + sum;
+      m = mn;
+      bf16x8_t pfr[2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        uint4 w;
+        w.x = pack2(sc[8 * s2 + 0], sc[8 * s2 + 1]);
+        w.y = pack2(sc[8 * s2 + 2], sc[8 * s2 + 3]);
+        w.z = pack2(sc[8 * s2 + 4], sc[8 * s2 + 5]);
+        w.w = pack2(sc[8 * s2 + 6], sc[8 * s2 + 7]);
+        pfr[s2] = __builtin_bit_cast(bf16x8_t, w);
+      }
+      const char* vbase = reinterpret_cast<const char*>(ks) + voff;
+      const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;  // wave-uniform: most tiles keep the max
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        if (rescale) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const char* a0 = vbase + (16 * s2) * pitchB + 64 * db;
+          const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0));
+          const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0 + 8 * pitchB));
+          const short8_t a8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a8), pfr[s2], o[db], 0, 0, 0);
+        }
+      }
+    }
+    if (j0 + MKT <= jhi) {
+      stash(ks0 + (cur ^ 1) * (MKT * KP));           // tile j0 + 32 (fetched one iteration ago) -> the other buffer
+      if (j0 + 2 * MKT <= jhi) fetch(j0 + 2 * MKT);  // in flight during the next tile's MFMAs
+    }
+  }
+  if (!rok) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  bf16_t* op = reinterpret_cast<bf16_t*>(a.out) + orow * R;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint2 w;
+      w.x = pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
+      w.y = pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
+      *reinterpret_cast<uint2*>(op + 32 * db + 8 * g + 4 * hh) = w;
+    }
+  }
+}
+
+template <int NDB, int NROT> hipError_t launch_mfma_rq(const LatentAttnArgs& a, hipStream_t s) {
+  static bool attr_set = false;
+  auto* fn = latent_attn_mfma_rq_kernel<NDB, NROT>;
+  const int kp = a.sh.rank + a.sh.rot_dim + 8;
+  const size_t lds = sizeof(bf16_t) * (size_t)2 * MKT * kp;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       64 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)(((int64_t)a.max_q * a.heads + 127) / 128), (unsigned)a.num_seqs);
+  hipLaunchKernelGGL(fn, grid, dim3(256), lds, s, a, kp);
+  return hipGetLastError();
+}
+
+// the register-query kernel exists for rank in {64, 128, 256} x rot_dim in {16, 32, 64}; unsplit steps only
+inline bool mfma_rq_ok(const LatentAttnArgs& a) {
+  const int r = a.sh.rank, t = a.sh.rot_dim;
+  return a.nsplit <= 1 && (int64_t)a.max_q * a.heads > 32 && (r == 64 || r == 128 || r == 256) &&
+         (t == 16 || t == 32 || t == 64);
+}
+
+template <int NDB> hipError_t launch_mfma_rq_rot(const LatentAttnArgs& a, hipStream_t s) {
+  switch (a.sh.rot_dim) {
+    case 16: return launch_mfma_rq<NDB, 1>(a, s);
+    case 32: return launch_mfma_rq<NDB, 2>(a, s);
+    case 64: return launch_mfma_rq<NDB, 4>(a, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_mfma_rq_any(const LatentAttnArgs& a, hipStream_t s) {
+  switch (a.sh.rank) {
+    case 64: return launch_mfma_rq_rot<2>(a, s);
+    case 128: return launch_mfma_rq_rot<4>(a, s);
+    case 256: return launch_mfma_rq_rot<8>(a, s);
+  }
+  return hipErrorInvalidValue;
+}
+
 hipError_t launch_mfma_any(const LatentAttnArgs& a, hipStream_t s) {
+  if (a.impl != 3 && mfma_rq_ok(a)) return launch_mfma_rq_any(a, s);
   // one wave per workgroup when a sequence brings at most 32 rows (decode steps): small LDS, many workgroups
   return (int64_t)a.max_q * a.heads <= 32 ? launch_mfma_ndb<1>(a, s) : launch_mfma_ndb<4>(a, s);
 }
@@ -496,7 +739,7 @@ hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s) {
       a.max_q < 1)
     return hipErrorInvalidValue;
   if (a.impl != 1 && mfma_ok(a)) return launch_mfma_any(a, s);
-  if (a.impl == 2) return hipErrorInvalidValue;  // the matrix-core form was demanded and does not apply
+  if (a.impl >= 2) return hipErrorInvalidValue;  // the matrix-core form was demanded and does not apply
   return a.f32 ? launch_bk<true>(a, s) : launch_bk<false>(a, s);
 }
 

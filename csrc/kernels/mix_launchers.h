@@ -27,6 +27,8 @@ hipError_t launch_gated_act(void* out, const void* gu, bool f32, int rows, int f
 // w [T, K] fp32 = the chosen scores (not renormalised), ids [T, K] int32
 hipError_t launch_route_sigmoid_topk(float* w, int* ids, const void* x, int64_t xstride, bool x_f32, const void* wr,
                                      bool wr_f32, int T, int H, int E, int K, hipStream_t s);
+// the same selection from fp32 logits z [T, E] computed elsewhere
+hipError_t launch_topk_sigmoid(float* w, int* ids, const float* z, int T, int E, int K, hipStream_t s);
 // xs[j] = w[sorted[j]] * x[sorted[j] / K]  (sorted == nullptr: j itself)
 hipError_t launch_gather_scaled(void* xs, const void* x, bool f32, const int* sorted, const float* w, int n, int K,
                                 int H, hipStream_t s);
@@ -68,7 +70,8 @@ struct LatentAttnArgs {
   float* ws_o;
   float* ws_ml;
   int nsplit, chunk;
-  int impl;               // 0: matrix cores where they apply, else the FMA form; 1: FMA form; 2: matrix cores or fail
+  int impl;               // 0: matrix cores where they apply, else the FMA form; 1: FMA form; 2: matrix cores or fail;
+                          // 3: as 2, but never the register-query variant (A/B)
 };
 hipError_t launch_latent_attn(const LatentAttnArgs& a, hipStream_t s);
 // whether launch_latent_attn would run the matrix-core kernel for these arguments (the split workspace is only

@@ -116,6 +116,31 @@ __global__ void __launch_bounds__(NT) route_sigmoid_topk_kernel(float* w_out, in
   }
 }
 
+// Selection alone, from logits already computed (a library fp32 GEMM for prompt-sized steps): one thread per token.
+__global__ void __launch_bounds__(NT) topk_sigmoid_kernel(float* w_out, int* id_out, const float* z, int T, int E,
+                                                         int K) {
+  const int t = blockIdx.x * NT + threadIdx.x;
+  if (t >= T) return;
+  const float* zr = z + (int64_t)t * E;
+  uint64_t taken[ROUTE_E_MAX / 64] = {0, 0, 0, 0};
+  for (int k = 0; k < K; ++k) {
+    int bi = -1;
+    float bv = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float v = zr[e];
+      if (v != v || ((taken[e >> 6] >> (e & 63)) & 1ull)) continue;
+      if (bi < 0 || v > bv) {
+        bv = v;
+        bi = e;
+      }
+    }
+    if (bi < 0) bi = 0;
+    taken[bi >> 6] |= 1ull << (bi & 63);
+    w_out[(int64_t)t * K + k] = 1.0f / (1.0f + expf(-bv));
+    id_out[(int64_t)t * K + k] = bi;
+  }
+}
+
 __global__ void __launch_bounds__(NT) gather_scaled_kernel(void* xs, const void* x, bool f32, const int* sorted,
                                                           const float* w, int K, int H) {
   const int64_t j = blockIdx.x;
@@ -206,6 +231,13 @@ hipError_t launch_route_sigmoid_topk(float* w, int* ids, const void* x, int64_t 
   if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E) return hipErrorInvalidValue;
   hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(T), dim3(NT), 0, s, w, ids, x, xstride, x_f32, wr, wr_f32, H, E,
                      K);
+  return hipGetLastError();
+}
+
+hipError_t launch_topk_sigmoid(float* w, int* ids, const float* z, int T, int E, int K, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(topk_sigmoid_kernel, dim3((T + NT - 1) / NT), dim3(NT), 0, s, w, ids, z, T, E, K);
   return hipGetLastError();
 }
 

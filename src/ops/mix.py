@@ -81,6 +81,9 @@ def gated_act(gu: torch.Tensor, kind: int = ACT_SILU, limit: float = 0.0, alpha:
     return out
 
 
+ROUTE_FUSED_MAX_T = 256  # up to here one fused launch computes the logits and selects (decode-sized steps)
+
+
 def route_sigmoid_topk(x: torch.Tensor, router: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """(w [T, k] fp32, ids [T, k] int32): the k experts with the largest sigmoid(x . router[e]) (fp32 logits) and
     those scores, not renormalised."""
@@ -89,7 +92,11 @@ def route_sigmoid_topk(x: torch.Tensor, router: torch.Tensor, k: int) -> Tuple[t
     t = x.shape[0]
     w = torch.empty(t, k, dtype=torch.float32, device=x.device)
     ids = torch.empty(t, k, dtype=torch.int32, device=x.device)
-    _kern().route_sigmoid_topk(w, ids, x, router.contiguous())
+    if t > ROUTE_FUSED_MAX_T:
+        # prompt-sized steps: the logits as one true-fp32 library GEMM, then the selection kernel
+        _kern().topk_sigmoid(w, ids, F.linear(x.float(), router.float()))
+    else:
+        _kern().route_sigmoid_topk(w, ids, x, router.contiguous())
     return w, ids
 
 
@@ -195,7 +202,8 @@ def latent_attn(q_lat: torch.Tensor, q: torch.Tensor, rot_off: int, cache: torch
     (q_lat . latent_j + q_rot . krot_j) * scale, softmax with exp(sink[h]) added to the denominator, and
     returns the weighted sum of the latent rows, [H, T, rank]. cu_q None: one query row per sequence.
     ``impl`` (GPU): 0 = the matrix-core kernel where it applies (bf16, rank % 32 == 0, rank <= 256,
-    rot_dim % 16 == 0), else the FMA kernel; 1 = the FMA kernel; 2 = the matrix-core kernel or an error."""
+    rot_dim % 16 == 0), else the FMA kernel; 1 = the FMA kernel; 2 = the matrix-core kernel or an error;
+    3 = as 2 but never its register-query variant (tests, A/B)."""
     if not q_lat.is_cuda:
         return ref.latent_attn(q_lat, q, rot_off, cache, block_tables, cu_q, ctx_lens, positions, sink, window, scale,
                                rot_dim, inv_freq)

@@ -177,12 +177,13 @@ def test_gated_activations(device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("top", [1, 2, 5])
-def test_routing_scores_not_renormalised(device, top):
+@pytest.mark.parametrize("tokens", [9, 300])   # fused logits + selection / library fp32 logits + selection kernel
+def test_routing_scores_not_renormalised(device, top, tokens):
     _need(device)
     from src import ops
 
     g = torch.Generator().manual_seed(2)
-    x, wr = torch.randn(9, 16, generator=g), torch.randn(5, 16, generator=g)
+    x, wr = torch.randn(tokens, 16, generator=g), torch.randn(5, 16, generator=g)
     w, ids = ops.route_sigmoid_topk(x.to(device), wr.to(device), top)
     ws, is_ = orc.route(x.double(), wr.double(), top)
     assert torch.equal(ids.cpu().long(), is_)
@@ -233,7 +234,8 @@ def _dense_latent_attn(q_lat, q_rot, rows, p, sink, window, scale):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rank,rot,heads,window", [(12, 4, 3, 37), (40, 8, 5, 0), (130, 6, 2, 129), (8, 2, 1, 1),
-                                                   (64, 16, 6, 37), (96, 0, 2, 0), (256, 32, 7, 129), (32, 16, 1, 16)])
+                                                   (64, 16, 6, 37), (96, 0, 2, 0), (256, 32, 7, 129), (32, 16, 1, 16),
+                                                   (128, 64, 9, 0), (256, 64, 2, 200)])
 def test_latent_cache_and_attention_ops(device, dtype, rank, rot, heads, window):
     """latent_kv_write + latent_attn over scattered pages, against a dense computation: one standout key per
     query placed far back, on a page border, just inside and just outside the window (the outside one must be
@@ -287,13 +289,18 @@ def test_latent_cache_and_attention_ops(device, dtype, rank, rot, heads, window)
         out1 = ops.latent_attn(q_lat.to(device), q.to(device), 5, cache, bt, cu, ctx_t, p.to(device), sink.to(device),
                                nq, window, scale, rot, inv, impl=1)
         assert (out.float() - out1.float()).abs().max() < 2e-2 * out1.float().abs().max()
+        # impl 3: the matrix-core kernel that keeps the queries in LDS (the one decode-sized steps and other
+        # rotary widths use), on the same prompt-sized step
+        out3 = ops.latent_attn(q_lat.to(device), q.to(device), 5, cache, bt, cu, ctx_t, p.to(device), sink.to(device),
+                               nq, window, scale, rot, inv, impl=3)
+        assert (out3.float() - out1.float()).abs().max() < 2e-2 * out1.float().abs().max()
     q_rot = orc.rotate_interleaved(q.view(nq, heads, qh)[:, :, 5:].double(), p, base, rot).transpose(0, 1)
     want = _dense_latent_attn(q_lat.double(), q_rot, rows, p, sink, window, scale)
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     assert (out.cpu().double() - want).abs().max() < tol * want.abs().max()
     # the sink takes weight: without it the outputs differ
     no_sink = _dense_latent_attn(q_lat.double(), q_rot, rows, p, None, window, scale)
-    assert (no_sink - want).abs().max() > 0.1 * want.abs().max()
+    assert (no_sink - want).abs().max() > 0.03 * want.abs().max()
     # decode form: one row per sequence, three "sequences" sharing the pages at different lengths
     lens = [ctx, ctx - 9, 17]
     qd = q[:3].to(device)
