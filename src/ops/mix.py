@@ -30,12 +30,25 @@ except Exception as e:  # pragma: no cover - depends on build state
     _CMIX_ERR = e
 
 
+def _load():
+    """Import the extension if it was not there when this module was first imported (built since, in place)."""
+    global _Cmix, _CMIX_ERR
+    if _Cmix is None:
+        try:
+            import importlib
+
+            _Cmix = importlib.import_module("src._Cmix")
+        except Exception as e:  # noqa: BLE001
+            _CMIX_ERR = e
+    return _Cmix
+
+
 def mix_available() -> bool:
-    return _Cmix is not None
+    return _load() is not None
 
 
 def _kern():
-    if _Cmix is None:
+    if _load() is None:
         raise RuntimeError(
             "HIP kernel extension src/_Cmix is not built or failed to load "
             f"({_CMIX_ERR!r}); run `python -m src._build --mix-only` (hipcc --offload-arch=gfx950)")
