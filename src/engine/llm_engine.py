@@ -577,6 +577,8 @@ class LLMEngine:
         plan, rows, base = [], [], 0
         for rid, toks, want in entries:
             toks = [int(x) for x in toks]
+            if not toks:  # a request named in a step without tokens neither runs nor is admitted
+                continue
             if toks and (min(toks) < 0 or max(toks) >= self.arch.vocab_size):
                 raise ValueError(f"token id outside [0, {self.arch.vocab_size})")
             seq = self.seqs.get(rid)
