@@ -230,23 +230,27 @@ __global__ void __launch_bounds__(64 * NW) latent_attn_mfma_kernel(LatentAttnArg
     }
     *reinterpret_cast<uint4*>(qs + r * KP + 8 * c) = v;
   }
-  for (int idx = tid; idx < ROWS * a.sh.rot_dim; idx += NT) {
-    const int r = idx / a.sh.rot_dim, dd = idx % a.sh.rot_dim, row = row0 + r;
-    float v = 0.f;
+  // one thread per interleaved pair (an odd last element passes unchanged); bf16 operands: the fast sin / cos
+  const int npair = (a.sh.rot_dim + 1) / 2;
+  for (int idx = tid; idx < ROWS * npair; idx += NT) {
+    const int r = idx / npair, i = idx % npair, row = row0 + r;
+    const bool two = 2 * i + 1 < a.sh.rot_dim;
+    float v0 = 0.f, v1 = 0.f;
     if (row < nrows) {
       const int64_t t = q0 + row / H;
       const int64_t qr = t * a.q_stride + (int64_t)(row % H) * a.q_hstride;
-      const int i = dd >> 1;
+      const float u = bf2f(qrot[qr + 2 * i]), w = two ? bf2f(qrot[qr + 2 * i + 1]) : 0.f;
+      v0 = u;
+      v1 = w;
       if (i < a.sh.rot_pairs) {
-        const float u = bf2f(qrot[qr + 2 * i]), w = bf2f(qrot[qr + 2 * i + 1]);
         float sn, cs;
-        sincosf((float)a.positions[t] * a.sh.inv_freq[i], &sn, &cs);
-        v = (dd & 1) ? w * cs + u * sn : u * cs - w * sn;
-      } else {
-        v = bf2f(qrot[qr + dd]);
+        __sincosf((float)a.positions[t] * a.sh.inv_freq[i], &sn, &cs);
+        v0 = u * cs - w * sn;
+        v1 = w * cs + u * sn;
       }
     }
-    qs[r * KP + R + dd] = f2bf(v);
+    qs[r * KP + R + 2 * i] = f2bf(v0);
+    if (two) qs[r * KP + R + 2 * i + 1] = f2bf(v1);
   }
 
   const bool wave_live = row0 + wave * 32 < nrows;
@@ -503,7 +507,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_rq_kernel(LatentAttnArgs
         const float u = bf2f(qp[2 * pr]), w = bf2f(qp[2 * pr + 1]);
         if (i < a.sh.rot_pairs) {
           float sn, cs;
-          sincosf((float)prow * a.sh.inv_freq[i], &sn, &cs);
+          __sincosf((float)prow * a.sh.inv_freq[i], &sn, &cs);
           f[2 * pr] = u * cs - w * sn;
           f[2 * pr + 1] = w * cs + u * sn;
         } else {

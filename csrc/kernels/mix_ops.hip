@@ -90,9 +90,25 @@ __global__ void __launch_bounds__(NT) route_sigmoid_topk_kernel(float* w_out, in
                                                                bool wr_f32, int H, int E, int K) {
   __shared__ float z[ROUTE_E_MAX];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // 16-byte loads where both rows allow them (bf16 x and router: 8 elements per lane and trip, independent trips)
+  const bool vec = !x_f32 && !wr_f32 && H % 8 == 0 && xstride % 8 == 0 &&
+                   (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wr) & 15) == 0;
   for (int e = wave; e < E; e += NT / 64) {
     float a = 0.f;
-    for (int c = lane; c < H; c += 64) a += ldv(x, (int64_t)t * xstride + c, x_f32) * ldv(wr, (int64_t)e * H + c, wr_f32);
+    if (vec) {
+      const uint4* xr = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + (int64_t)t * xstride);
+      const uint4* wp = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(wr) + (int64_t)e * H);
+      for (int c = lane; c < H / 8; c += 64) {
+        float xf[8], wf[8];
+        unpack8(xr[c], xf);
+        unpack8(wp[c], wf);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a += xf[q] * wf[q];
+      }
+    } else {
+      for (int c = lane; c < H; c += 64)
+        a += ldv(x, (int64_t)t * xstride + c, x_f32) * ldv(wr, (int64_t)e * H + c, wr_f32);
+    }
     a = wave_sum(a);
     if (lane == 0) z[e] = a;
   }
