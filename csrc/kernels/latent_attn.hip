@@ -179,6 +179,7 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(LatentAttnArgs a, int 
 // writes its unnormalised O, running max and sum to a workspace, and latent_attn_merge_kernel combines them;
 // the sink enters split 0 only.
 constexpr int MKT = 32;
+constexpr int BT_LDS_MAX = 2048;  // block-table entries staged per workgroup (else read from global memory)
 typedef __attribute__((address_space(3))) short4_t lds_short4;
 typedef __attribute__((ext_vector_type(8))) short short8_t;
 
@@ -189,11 +190,22 @@ __global__ void __launch_bounds__(64 * NW) latent_attn_mfma_kernel(LatentAttnArg
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [ROWS][KP]
   bf16_t* ks = qs + ROWS * KP;                                // [MKT][KP]
-  const int s = blockIdx.y, z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  // unsplit steps: XCD k (workgroups are dealt round-robin by linear id) takes a contiguous eighth of the
+  // sequence-major tile list, so one sequence's cache rows stay in one L2
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (gridDim.z == 1) {
+    const unsigned total = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
+    if (total % 8 == 0) {
+      const unsigned nl = (lin % 8) * (total / 8) + lin / 8;
+      bx = (int)(nl % gridDim.x);
+      by = (int)(nl / gridDim.x);
+    }
+  }
+  const int s = by, z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
   const int H = a.heads, R = a.sh.rank, Dk = a.sh.rank + a.sh.rot_dim;
   const int q0 = a.cu_q ? a.cu_q[s] : s;
   const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
-  const int nrows = nq * H, row0 = blockIdx.x * ROWS;
+  const int nrows = nq * H, row0 = bx * ROWS;
   if (row0 >= nrows) return;
   const int ctx = a.ctx_lens[s];
   const int last_row = min(row0 + ROWS, nrows) - 1;
@@ -268,19 +280,28 @@ __global__ void __launch_bounds__(64 * NW) latent_attn_mfma_kernel(LatentAttnArg
 
   const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
   const int kch = Dk / 8, nkk = Dk / 16, nchunks = MKT * kch;
+  // block-table entries of this workgroup's key range in LDS (visible after the loop's first barrier; the first
+  // tile's loads read the table from global memory)
+  int* btl = reinterpret_cast<int*>(ks + MKT * KP);
+  const int b_lo = jlo / a.block_size, nbt = jhi / a.block_size - b_lo + 1;
+  const bool bt_lds = nbt <= BT_LDS_MAX;
+  if (bt_lds)
+    for (int u = tid; u < nbt; u += NT) btl[u] = bt[b_lo + u];
   uint4 pf[NPF];
-  auto fetch = [&](int j0) {
+  auto fetch = [&](int j0, bool lds) {
 #pragma unroll
     for (int u = 0; u < NPF; ++u) {
       const int idx = tid + u * NT;
       const int k = idx / kch, c = idx % kch, j = j0 + k;
       pf[u] = make_uint4(0, 0, 0, 0);
-      if (idx < nchunks && j <= jhi)
-        pf[u] = *reinterpret_cast<const uint4*>(
-            cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
+      if (idx < nchunks && j <= jhi) {
+        const int jb = j / a.block_size;
+        const int64_t blk = lds ? btl[jb - b_lo] : bt[jb];
+        pf[u] = *reinterpret_cast<const uint4*>(cache + (blk * a.block_size + (j - jb * a.block_size)) * Dk + 8 * c);
+      }
     }
   };
-  fetch(jlo);
+  fetch(jlo, false);
   const int pitchB = KP * 2;
   const int g16 = lane >> 4, i16 = lane & 15;
   const char* vbase = reinterpret_cast<const char*>(ks) + (4 * hh + (i16 >> 2)) * pitchB +
@@ -293,7 +314,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attn_mfma_kernel(LatentAttnArg
       if (idx < nchunks) *reinterpret_cast<uint4*>(ks + (idx / kch) * KP + 8 * (idx % kch)) = pf[u];
     }
     __syncthreads();
-    if (j0 + MKT <= jhi) fetch(j0 + MKT);  // in flight while this tile is computed
+    if (j0 + MKT <= jhi) fetch(j0 + MKT, bt_lds);  // in flight while this tile is computed
     if (!wave_live) continue;
     f32x16_t sc;
 #pragma unroll
@@ -404,7 +425,9 @@ __global__ void __launch_bounds__(256) latent_attn_merge_kernel(bf16_t* out, con
   }
 }
 
-inline size_t mfma_lds_bytes(int kp, int nw) { return sizeof(bf16_t) * (size_t)(32 * nw + MKT) * kp; }
+inline size_t mfma_lds_bytes(int kp, int nw) {
+  return sizeof(bf16_t) * (size_t)(32 * nw + MKT) * kp + sizeof(int) * BT_LDS_MAX;
+}
 
 template <int NDB, int NW> hipError_t launch_mfma(const LatentAttnArgs& a, hipStream_t s) {
   static bool attr_set = false;
@@ -458,12 +481,24 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_rq_kernel(LatentAttnArgs
   constexpr int NPF = (NCH + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   bf16_t* ks0 = reinterpret_cast<bf16_t*>(smem_raw);          // 2 x [MKT][KP]
-  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  // Workgroups are dealt to the 8 XCDs round-robin by their linear id, and each XCD has its own L2: renumber so
+  // that XCD k runs a contiguous eighth of the (sequence-major) tile list — the row tiles of one sequence share
+  // that sequence's cache rows in ONE L2 instead of streaming every sequence through all eight
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    const unsigned total = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
+    if (total % 8 == 0) {
+      const unsigned nl = (lin % 8) * (total / 8) + lin / 8;
+      bx = (int)(nl % gridDim.x);
+      by = (int)(nl / gridDim.x);
+    }
+  }
+  const int s = by, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
   const int H = a.heads;
   constexpr int R = 32 * NDB, Dk = R + 16 * NROT;
   const int q0 = a.cu_q ? a.cu_q[s] : s;
   const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
-  const int nrows = nq * H, row0 = blockIdx.x * 128;
+  const int nrows = nq * H, row0 = bx * 128;
   if (row0 >= nrows) return;
   const int ctx = a.ctx_lens[s];
   const int last_row = min(row0 + 128, nrows) - 1;
@@ -530,7 +565,16 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_rq_kernel(LatentAttnArgs
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
 
+  // the block-table entries of this workgroup's key range, staged in LDS: a key tile's loads then depend on an
+  // LDS read, not on a second global round trip
   const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
+  int* btl = reinterpret_cast<int*>(ks0 + 2 * MKT * KP);
+  const int b_lo = jlo / a.block_size, nbt = jhi / a.block_size - b_lo + 1;
+  const bool bt_lds = nbt <= BT_LDS_MAX;
+  if (bt_lds) {
+    for (int u = tid; u < nbt; u += NT) btl[u] = bt[b_lo + u];
+    __syncthreads();
+  }
   uint4 pf[NPF];
   auto fetch = [&](int j0) {
 #pragma unroll
@@ -538,9 +582,11 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_rq_kernel(LatentAttnArgs
       const int idx = tid + u * NT;
       const int k = idx / KCH, c = idx % KCH, j = j0 + k;
       pf[u] = make_uint4(0, 0, 0, 0);
-      if (idx < NCH && j <= jhi)
-        pf[u] = *reinterpret_cast<const uint4*>(
-            cache + ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * Dk + 8 * c);
+      if (idx < NCH && j <= jhi) {
+        const int jb = j / a.block_size;
+        const int64_t blk = bt_lds ? btl[jb - b_lo] : bt[jb];
+        pf[u] = *reinterpret_cast<const uint4*>(cache + (blk * a.block_size + (j - jb * a.block_size)) * Dk + 8 * c);
+      }
     }
   };
   auto stash = [&](bf16_t* ks) {
@@ -653,7 +699,7 @@ template <int NDB, int NROT> hipError_t launch_mfma_rq(const LatentAttnArgs& a, 
   static bool attr_set = false;
   auto* fn = latent_attn_mfma_rq_kernel<NDB, NROT>;
   const int kp = a.sh.rank + a.sh.rot_dim + 8;
-  const size_t lds = sizeof(bf16_t) * (size_t)2 * MKT * kp;
+  const size_t lds = sizeof(bf16_t) * (size_t)2 * MKT * kp + sizeof(int) * BT_LDS_MAX;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        64 * 1024);
