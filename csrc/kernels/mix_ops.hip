@@ -51,11 +51,41 @@ __global__ void __launch_bounds__(NT) rms_norm_ext_kernel(void* out, int64_t ost
   }
 }
 
+__device__ __forceinline__ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, void* act, const void* y,
                                                                int64_t ystride, bool y_f32, const void* w, bool w_f32,
                                                                bool unit, float eps, int n) {
   __shared__ float red[NT / 64];
   const int64_t r = blockIdx.x;
+  // bf16 rows of a multiple of 8 columns: 16-byte loads and stores, 8 columns per thread and trip
+  if (!y_f32 && !w_f32 && n % 8 == 0 && ystride % 8 == 0 && aligned16(y) && aligned16(w) && aligned16(resid) &&
+      (act == nullptr || aligned16(act))) {
+    const uint4* yr = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(y) + r * ystride);
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < n / 8; c += NT) {
+      float f[8];
+      unpack8(yr[c], f);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) ss += f[q] * f[q];
+    }
+    ss = block_sum<NT>(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)n + eps);
+    float4* rr = reinterpret_cast<float4*>(resid + r * n);
+    for (int c = threadIdx.x; c < n / 8; c += NT) {
+      float f[8], g[8];
+      unpack8(yr[c], f);
+      unpack8(reinterpret_cast<const uint4*>(w)[c], g);
+      float4 a0 = rr[2 * c], a1 = rr[2 * c + 1];
+      float o[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] += f[q] * rs * (unit ? g[q] + 1.0f : g[q]);
+      rr[2 * c] = make_float4(o[0], o[1], o[2], o[3]);
+      rr[2 * c + 1] = make_float4(o[4], o[5], o[6], o[7]);
+      if (act) reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(act) + r * n)[c] = pack8(o);
+    }
+    return;
+  }
   const float rs = row_rs(y, r * ystride, y_f32, n, eps, red);
   for (int c = threadIdx.x; c < n; c += NT) {
     float g = w ? ldv(w, c, w_f32) : 1.0f;
@@ -66,20 +96,32 @@ __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, vo
   }
 }
 
+__device__ __forceinline__ float gate1(float g, float u, int kind, float limit, float alpha) {
+  if (kind == 0) return g / (1.0f + expf(-g)) * u;
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
+
 __global__ void __launch_bounds__(NT) gated_act_kernel(void* out, const void* gu, bool f32, int f, int kind,
                                                       float limit, float alpha) {
   const int64_t r = blockIdx.x;
-  for (int c = threadIdx.x; c < f; c += NT) {
-    float g = ldv(gu, r * 2 * f + c, f32), u = ldv(gu, r * 2 * f + f + c, f32), v;
-    if (kind == 0) {
-      v = g / (1.0f + expf(-g)) * u;
-    } else {
-      g = fminf(g, limit);
-      u = fminf(fmaxf(u, -limit), limit);
-      v = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  if (!f32 && f % 8 == 0 && aligned16(gu) && aligned16(out)) {
+    const uint4* gp = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(gu) + r * 2 * f);
+    const uint4* up = gp + f / 8;
+    uint4* op = reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(out) + r * f);
+    for (int c = threadIdx.x; c < f / 8; c += NT) {
+      float g[8], u[8], o[8];
+      unpack8(gp[c], g);
+      unpack8(up[c], u);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] = gate1(g[q], u[q], kind, limit, alpha);
+      op[c] = pack8(o);
     }
-    stv(out, r * f + c, f32, v);
+    return;
   }
+  for (int c = threadIdx.x; c < f; c += NT)
+    stv(out, r * f + c, f32, gate1(ldv(gu, r * 2 * f + c, f32), ldv(gu, r * 2 * f + f + c, f32), kind, limit, alpha));
 }
 
 constexpr int ROUTE_E_MAX = 256;
@@ -163,12 +205,42 @@ __global__ void __launch_bounds__(NT) gather_scaled_kernel(void* xs, const void*
   const int flat = sorted ? sorted[j] : (int)j;
   const int64_t t = flat / K;
   const float wk = w[flat];
+  if (!f32 && H % 8 == 0 && aligned16(x) && aligned16(xs)) {
+    const uint4* xp = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + t * H);
+    uint4* op = reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(xs) + j * H);
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float v[8];
+      unpack8(xp[c], v);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] *= wk;
+      op[c] = pack8(v);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < H; c += NT) stv(xs, j * H + c, f32, wk * ldv(x, t * H + c, f32));
 }
 
 __global__ void __launch_bounds__(NT) combine_sum_kernel(float* out, const void* ys, bool f32, const int* pos,
                                                         const void* extra, int K, int H) {
   const int64_t t = blockIdx.x;
+  if (!f32 && H % 8 == 0 && aligned16(ys) && aligned16(out) && (extra == nullptr || aligned16(extra))) {
+    const bf16_t* yb = reinterpret_cast<const bf16_t*>(ys);
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (extra) unpack8(reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(extra) + t * H)[c], a);
+      for (int k = 0; k < K; ++k) {
+        const int64_t j = pos ? pos[t * K + k] : t * K + k;
+        float v[8];
+        unpack8(reinterpret_cast<const uint4*>(yb + j * H)[c], v);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a[q] += v[q];
+      }
+      float4* op = reinterpret_cast<float4*>(out + t * H);
+      op[2 * c] = make_float4(a[0], a[1], a[2], a[3]);
+      op[2 * c + 1] = make_float4(a[4], a[5], a[6], a[7]);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < H; c += NT) {
     float a = extra ? ldv(extra, t * H + c, f32) : 0.f;
     for (int k = 0; k < K; ++k) {

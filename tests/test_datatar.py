@@ -173,6 +173,13 @@ def test_gated_activations(device):
     ac, bc = a.clamp(max=lim), b.clamp(-lim, lim)
     assert (y - ac * torch.sigmoid(1.702 * ac) * (bc + 1)).abs().max() < 1e-5
     assert float(a.min()) < -lim and float(a.max()) > lim   # the gate is clamped above only
+    # bf16 rows of a multiple of 8 columns (the 16-byte path on the GPU)
+    gb = (torch.randn(5, 2 * 16, generator=g) * 2).to(torch.bfloat16)
+    ab, bb = gb[:, :16].double(), gb[:, 16:].double()
+    for kind, want in ((ops.ACT_SILU, ab * torch.sigmoid(ab) * bb),
+                       (ops.ACT_CLAMPED, ab.clamp(max=lim) * torch.sigmoid(1.702 * ab.clamp(max=lim)) * (bb.clamp(-lim, lim) + 1))):
+        y = ops.gated_act(gb.to(device), kind, lim, 1.702).cpu().double()
+        assert (y - want).abs().max() < 1e-2 * want.abs().max()
 
 
 @pytest.mark.parametrize("device", DEVICES)
