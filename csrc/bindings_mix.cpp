@@ -171,6 +171,62 @@ void latent_kv_write(Tensor cache, Tensor kv, Tensor w, Tensor positions, Tensor
                                      latent_shape(rank, rot_dim, inv_freq), (float)eps, cur_stream()));
 }
 
+// p [T, q_rank + rank + rot_dim]: cq [T, q_rank] = rmsnorm(p[:, :q_rank]) * wq; cache rows from p[:, q_rank:]
+void latent_qkv_prep(Tensor cq, Tensor cache, Tensor p, Tensor wq, Tensor wkv, Tensor positions, Tensor slots,
+                     int64_t rank, int64_t rot_dim, Tensor inv_freq, double eps) {
+  check_rows(p, "p");
+  const bool f = is_f32(p, "p"), wf = is_f32(wq, "wq");
+  const int64_t q_rank = p.size(1) - rank - rot_dim;
+  TORCH_CHECK(q_rank >= 1, "p narrower than the cache row");
+  TORCH_CHECK(is_f32(cq, "cq") == f && cq.is_contiguous() && cq.dim() == 2 && cq.size(0) == p.size(0) &&
+                  cq.size(1) == q_rank,
+              "cq [T, q_rank], dtype of p");
+  TORCH_CHECK(is_f32(cache, "cache") == f && cache.is_contiguous() && cache.dim() == 3 &&
+                  cache.size(2) == rank + rot_dim,
+              "cache [blocks, block_size, rank + rot_dim], dtype of p");
+  TORCH_CHECK(is_f32(wkv, "wkv") == wf && wq.is_contiguous() && wkv.is_contiguous() && wq.numel() == q_rank &&
+                  wkv.numel() == rank,
+              "wq [q_rank], wkv [rank], one dtype");
+  check_i(positions, at::kLong, "positions");
+  check_i(slots, at::kLong, "slots");
+  TORCH_CHECK(positions.numel() >= p.size(0) && slots.numel() >= p.size(0), "positions / slots [T]");
+  HIP_OK(die::launch_latent_qkv_prep(cq.data_ptr(), p.data_ptr(), p.stride(0), f, (int)q_rank, wq.data_ptr(),
+                                     wkv.data_ptr(), wf, cache.data_ptr(), positions.data_ptr<int64_t>(),
+                                     slots.data_ptr<int64_t>(), (int)p.size(0), latent_shape(rank, rot_dim, inv_freq),
+                                     (float)eps, cur_stream()));
+}
+
+void combine_post_norm(Tensor resid, OptTensor act, Tensor ys, OptTensor pos, OptTensor extra, int64_t topk, Tensor w,
+                       bool unit_offset, double eps) {
+  const bool f = is_f32(ys, "ys"), wf = is_f32(w, "w");
+  check_i(resid, at::kFloat, "resid");
+  TORCH_CHECK(resid.dim() == 2 && ys.dim() == 2 && ys.is_contiguous() && ys.size(1) == resid.size(1) &&
+                  ys.size(0) == resid.size(0) * topk && w.is_contiguous() && w.numel() == resid.size(1),
+              "combine_post_norm shapes");
+  const int* pp = nullptr;
+  if (pos.has_value()) {
+    check_i(*pos, at::kInt, "pos");
+    TORCH_CHECK(pos->numel() == ys.size(0), "pos [T * K]");
+    pp = pos->data_ptr<int>();
+  }
+  const void* ep = nullptr;
+  if (extra.has_value()) {
+    TORCH_CHECK(is_f32(*extra, "extra") == f && extra->is_contiguous() && extra->sizes() == resid.sizes(),
+                "extra: same dtype as ys, shape of resid");
+    ep = extra->data_ptr();
+  }
+  void* ap = nullptr;
+  if (act.has_value()) {
+    TORCH_CHECK(act->is_cuda() && act->scalar_type() == at::kBFloat16 && act->is_contiguous() &&
+                    act->sizes() == resid.sizes(),
+                "act must be a contiguous bf16 tensor of the residual's shape");
+    ap = act->data_ptr();
+  }
+  HIP_OK(die::launch_combine_post_norm(resid.data_ptr<float>(), ap, ys.data_ptr(), f, pp, ep, (int)resid.size(0),
+                                       (int)topk, (int)resid.size(1), w.data_ptr(), wf, unit_offset, (float)eps,
+                                       cur_stream()));
+}
+
 // out, q_lat [H, T, rank]; q [T, H * qh] whose head h keeps its rotary part at [h * qh + rot_off, + rot_dim)
 void latent_attn(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cache, Tensor block_tables,
                  OptTensor cu_q, Tensor ctx_lens, Tensor positions, OptTensor sink, int64_t max_q, int64_t window,
@@ -279,5 +335,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("combine_sum", &combine_sum);
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_attn", &latent_attn);
+  m.def("latent_qkv_prep", &latent_qkv_prep);
+  m.def("combine_post_norm", &combine_post_norm);
   m.def("moe_align", &moe_align);
 }

@@ -47,6 +47,16 @@ hipError_t launch_latent_kv_write(void* cache, const void* kv, int64_t kvstride,
                                   const int64_t* positions, const int64_t* slots, int T, LatentShape sh, float eps,
                                   hipStream_t s);
 
+// p [T, q_rank + rank + rot_dim] (row stride pstride): cq[t] = rmsnorm(p[t, :q_rank]) * wq and the cache row of
+// token t from p[t, q_rank:], as launch_latent_kv_write — one launch for both
+hipError_t launch_latent_qkv_prep(void* cq, const void* p, int64_t pstride, bool f32, int q_rank, const void* wq,
+                                  const void* wkv, bool w_f32, void* cache, const int64_t* positions,
+                                  const int64_t* slots, int T, LatentShape sh, float eps, hipStream_t s);
+// resid[t] (fp32) += rmsnorm(sum_k ys[pos[t * K + k]] + extra[t]) * (w or 1 + w); act[t] (optional, bf16) = resid[t]
+hipError_t launch_combine_post_norm(float* resid, void* act, const void* ys, bool f32, const int* pos,
+                                    const void* extra, int T, int K, int H, const void* w, bool w_f32,
+                                    bool unit_offset, float eps, hipStream_t s);
+
 struct LatentAttnArgs {
   void* out;              // [H, T, rank] latent-space attention output
   const void* q_lat;      // [H, T, rank] queries projected into the latent space

@@ -251,11 +251,9 @@ __global__ void __launch_bounds__(NT) combine_sum_kernel(float* out, const void*
   }
 }
 
-__global__ void __launch_bounds__(NT) latent_kv_write_kernel(void* cache, const void* kv, int64_t kvstride, bool f32,
-                                                            const void* w, bool w_f32, const int64_t* positions,
-                                                            const int64_t* slots, LatentShape sh, float eps) {
-  __shared__ float red[NT / 64];
-  const int64_t t = blockIdx.x;
+__device__ __forceinline__ void kv_write_row(void* cache, const void* kv, int64_t kvstride, bool f32, const void* w,
+                                             bool w_f32, const int64_t* positions, const int64_t* slots,
+                                             const LatentShape& sh, float eps, int64_t t, float* red) {
   const int64_t slot = slots[t];
   if (slot < 0) return;  // uniform per workgroup
   const int64_t src = t * kvstride, dst = slot * (int64_t)(sh.rank + sh.rot_dim);
@@ -280,6 +278,97 @@ __global__ void __launch_bounds__(NT) latent_kv_write_kernel(void* cache, const 
       stv(cache, dst + sh.rank + c0, f32, u);
       stv(cache, dst + sh.rank + c0 + 1, f32, v);
     }
+  }
+}
+
+__global__ void __launch_bounds__(NT) latent_kv_write_kernel(void* cache, const void* kv, int64_t kvstride, bool f32,
+                                                            const void* w, bool w_f32, const int64_t* positions,
+                                                            const int64_t* slots, LatentShape sh, float eps) {
+  __shared__ float red[NT / 64];
+  kv_write_row(cache, kv, kvstride, f32, w, w_f32, positions, slots, sh, eps, blockIdx.x, red);
+}
+
+// Both consumers of the fused down-projection p = [query latent | kv latent | shared rotary key] in one launch:
+// blockIdx.y == 0 norms the query latent (plain weight) into cq, blockIdx.y == 1 writes the cache row.
+__global__ void __launch_bounds__(NT) latent_qkv_prep_kernel(void* cq, const void* p, int64_t pstride, bool f32,
+                                                            int q_rank, const void* wq, const void* wkv, bool w_f32,
+                                                            void* cache, const int64_t* positions,
+                                                            const int64_t* slots, LatentShape sh, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  if (blockIdx.y == 0) {
+    const float rs = row_rs(p, t * pstride, f32, q_rank, eps, red);
+    for (int c = threadIdx.x; c < q_rank; c += NT)
+      stv(cq, t * q_rank + c, f32, ldv(p, t * pstride + c, f32) * rs * ldv(wq, c, w_f32));
+  } else {
+    const char* kv = reinterpret_cast<const char*>(p) + (size_t)q_rank * (f32 ? 4 : 2);
+    kv_write_row(cache, kv, pstride, f32, wkv, w_f32, positions, slots, sh, eps, t, red);
+  }
+}
+
+// resid[t] (fp32) += rmsnorm(sum_k ys[pos[t, k]] + extra[t]) * (w | 1 + w); act[t] (optional, bf16) = resid[t].
+// The expert sum is formed twice (statistics, then the update) instead of round-tripping through memory.
+__global__ void __launch_bounds__(NT) combine_post_norm_kernel(float* resid, void* act, const void* ys, bool f32,
+                                                              const int* pos, const void* extra, int K, int H,
+                                                              const void* w, bool w_f32, bool unit, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  if (!f32 && !w_f32 && H % 8 == 0 && aligned16(ys) && aligned16(resid) && aligned16(w) &&
+      (extra == nullptr || aligned16(extra)) && (act == nullptr || aligned16(act))) {
+    const bf16_t* yb = reinterpret_cast<const bf16_t*>(ys);
+    auto sum8 = [&](int c, float* a) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) a[q] = 0.f;
+      if (extra) unpack8(reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(extra) + t * H)[c], a);
+      for (int k = 0; k < K; ++k) {
+        float v[8];
+        unpack8(reinterpret_cast<const uint4*>(yb + (int64_t)(pos ? pos[t * K + k] : t * K + k) * H)[c], v);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a[q] += v[q];
+      }
+    };
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float a[8];
+      sum8(c, a);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) ss += a[q] * a[q];
+    }
+    ss = block_sum<NT>(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)H + eps);
+    float4* rr = reinterpret_cast<float4*>(resid + t * H);
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float a[8], g[8];
+      sum8(c, a);
+      unpack8(reinterpret_cast<const uint4*>(w)[c], g);
+      const float4 r0 = rr[2 * c], r1 = rr[2 * c + 1];
+      float o[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] += a[q] * rs * (unit ? g[q] + 1.0f : g[q]);
+      rr[2 * c] = make_float4(o[0], o[1], o[2], o[3]);
+      rr[2 * c + 1] = make_float4(o[4], o[5], o[6], o[7]);
+      if (act) reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(act) + t * H)[c] = pack8(o);
+    }
+    return;
+  }
+  auto sum_at = [&](int c) {
+    float a = extra ? ldv(extra, t * H + c, f32) : 0.f;
+    for (int k = 0; k < K; ++k) a += ldv(ys, (int64_t)(pos ? pos[t * K + k] : t * K + k) * H + c, f32);
+    return a;
+  };
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += NT) {
+    const float a = sum_at(c);
+    ss += a * a;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float rs = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += NT) {
+    float g = ldv(w, c, w_f32);
+    if (unit) g += 1.0f;
+    const float v = resid[t * H + c] + sum_at(c) * rs * g;
+    resid[t * H + c] = v;
+    if (act) reinterpret_cast<bf16_t*>(act)[t * H + c] = f2bf(v);
   }
 }
 
@@ -340,6 +429,26 @@ hipError_t launch_combine_sum(float* out, const void* ys, bool f32, const int* p
                               int H, hipStream_t s) {
   if (T == 0) return hipSuccess;
   hipLaunchKernelGGL(combine_sum_kernel, dim3(T), dim3(NT), 0, s, out, ys, f32, pos, extra, K, H);
+  return hipGetLastError();
+}
+
+hipError_t launch_latent_qkv_prep(void* cq, const void* p, int64_t pstride, bool f32, int q_rank, const void* wq,
+                                  const void* wkv, bool w_f32, void* cache, const int64_t* positions,
+                                  const int64_t* slots, int T, LatentShape sh, float eps, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (q_rank <= 0 || sh.rank <= 0 || sh.rot_dim < 0 || sh.rot_pairs * 2 > sh.rot_dim) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(latent_qkv_prep_kernel, dim3(T, 2), dim3(NT), 0, s, cq, p, pstride, f32, q_rank, wq, wkv, w_f32,
+                     cache, positions, slots, sh, eps);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_post_norm(float* resid, void* act, const void* ys, bool f32, const int* pos,
+                                    const void* extra, int T, int K, int H, const void* w, bool w_f32,
+                                    bool unit_offset, float eps, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (H <= 0 || K < 1) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(combine_post_norm_kernel, dim3(T), dim3(NT), 0, s, resid, act, ys, f32, pos, extra, K, H, w, w_f32,
+                     unit_offset, eps);
   return hipGetLastError();
 }
 

@@ -247,9 +247,9 @@ class LatentAttentionMixer:
         s = self.spec
         t = a.shape[0]
         p = mix.linear(a, self.dqkv)
-        q = mix.linear(mix.rms_norm_ext(p[:, : s.q_rank], self.dq_norm, eps), self.uq)
-        mix.latent_kv_write(cache, p[:, s.q_rank:], self.dkv_norm, positions, meta.slot_mapping, s.kv_rank, s.rot_dim,
-                            self.inv_freq, eps)
+        cq = mix.latent_qkv_prep(p, s.q_rank, self.dq_norm, self.dkv_norm, cache, positions, meta.slot_mapping,
+                                 s.kv_rank, s.rot_dim, self.inv_freq, eps)
+        q = mix.linear(cq, self.uq)
         q_lat = torch.bmm(q.view(t, s.heads, s.dim + s.rot_dim)[:, :, : s.dim].transpose(0, 1), self.uk)
         o_lat = mix.latent_attn(q_lat, q, s.dim, cache, meta.block_tables, meta.cu_q if meta.is_prefill else None,
                                 meta.ctx_lens, positions, self.sink, meta.max_q_len if meta.is_prefill else 1,
@@ -489,19 +489,23 @@ class DatatarLM:
                 meta.kv_hook(li)
             f = self.arch.layers[li].mlp
             if f is not None:
-                mix.post_norm_residual(resid, self._mlp(lw, f, act), lw.norm2, eps, True, act=act_out)
+                y = self._mlp(lw, f, act, post_norm=(resid, lw.norm2, eps, True, act_out))
+                if y is not None:
+                    mix.post_norm_residual(resid, y, lw.norm2, eps, True, act=act_out)
             if layer_hook is not None:
                 layer_hook(li, resid)
         return mix.rms_norm_ext(resid, self.norm, eps, True, out_dtype=self.dtype)
 
-    def _mlp(self, lw: MixLayerWeights, f: MlpSpec, a: torch.Tensor) -> torch.Tensor:
+    def _mlp(self, lw: MixLayerWeights, f: MlpSpec, a: torch.Tensor, post_norm=None) -> Optional[torch.Tensor]:
+        """The feed-forward's output, or None when it was already added into the residual (``post_norm``: the MoE's
+        expert sum and its post-norm are one launch)."""
         if f.kind == "dense":
             return mix.linear(mix.gated_act(mix.linear(a, lw.gate_up), mix.ACT_CLAMPED, f.limit, GATE_ALPHA), lw.down)
         w, ids = mix.route_sigmoid_topk(a, lw.router, f.top)
         shared = None
         if lw.shared_gate_up is not None:
             shared = mix.linear(mix.gated_act(mix.linear(a, lw.shared_gate_up), mix.ACT_SILU), lw.shared_down)
-        return mix.moe_input_scaled(a, lw.w13, lw.w2, w, ids, extra=shared)
+        return mix.moe_input_scaled(a, lw.w13, lw.w2, w, ids, extra=shared, post_norm=post_norm)
 
     def compute_logits(self, hidden: torch.Tensor, argmax_parts=None) -> torch.Tensor:
         """fp32 logits [rows, vocab] = head(hidden) * logit_scale."""

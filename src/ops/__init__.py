@@ -923,5 +923,6 @@ def _moe_down_wr(hdim: int, inter: int) -> int:
 
 
 # dtype-generic ops (bf16 / fp32 storage) of the src/_Cmix extension
-from .mix import (ACT_CLAMPED, ACT_SILU, gated_act, latent_attn, latent_kv_write, mix_available,  # noqa: E402,F401
+from .mix import (ACT_CLAMPED, ACT_SILU, gated_act, latent_attn, latent_kv_write, latent_qkv_prep,  # noqa: E402,F401
+                  mix_available,
                   moe_input_scaled, post_norm_residual, rms_norm_ext, rope_inv_freq, route_sigmoid_topk)

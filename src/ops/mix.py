@@ -131,11 +131,19 @@ MOE_BMM_MAX_ROWS = 64
 
 
 def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: torch.Tensor, ids: torch.Tensor,
-                     extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     extra: Optional[torch.Tensor] = None, post_norm=None) -> Optional[torch.Tensor]:
     """out[t] (fp32) = sum_j expert_{ids[t, j]}(w[t, j] * x[t]) (+ extra[t]); expert(z) = W2 (silu(W1 z) * (W3 z))
-    with w13 [E, 2f, H] = [W1; W3] and w2 [E, H, f]. The routing weight multiplies the expert's INPUT."""
+    with w13 [E, 2f, H] = [W1; W3] and w2 [E, H, f]. The routing weight multiplies the expert's INPUT.
+    ``post_norm`` = (resid fp32 [T, H], norm weight, eps, unit_offset, act or None): instead of returning the sum,
+    add its RMS-normalised form into ``resid`` (and refresh ``act``) in the same launch that forms it —
+    :func:`post_norm_residual` fused with the expert sum; returns None."""
     if not x.is_cuda:
-        return ref.moe_input_scaled(x, w13, w2, w, ids, extra)
+        out = ref.moe_input_scaled(x, w13, w2, w, ids, extra)
+        if post_norm is None:
+            return out
+        resid, nw, eps, unit, act = post_norm
+        post_norm_residual(resid, out, nw, eps, unit, act=act)
+        return None
     kern = _kern()
     t, h = x.shape
     k = ids.shape[1]
@@ -143,8 +151,17 @@ def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: to
     e = w13.shape[0]
     x = x.contiguous()
     w = w.contiguous()
-    out = torch.empty(t, h, dtype=torch.float32, device=x.device)
     xs = torch.empty(n, h, dtype=x.dtype, device=x.device)
+
+    def finish(ys, pos):
+        if post_norm is not None:
+            resid, nw, eps, unit, act = post_norm
+            kern.combine_post_norm(resid, act, ys, pos, extra, k, nw, unit, eps)
+            return None
+        out = torch.empty(t, h, dtype=torch.float32, device=x.device)
+        kern.combine_sum(out, ys, pos, extra, k)
+        return out
+
     if x.dtype == torch.bfloat16 and t <= 128:
         # decode-sized steps: the framework's expert-streaming grouped GEMM (every routed expert's weights
         # streamed once, SiLU * up fused; no host read, hipGraph-capturable) on the scaled, expert-sorted rows
@@ -164,15 +181,13 @@ def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: to
             none = ops._NO_ROWS(x.device)
             ck.gemm_decode_grouped(a, xs, w13, offsets, 1, wr1, kc1, none, 1, t, 1)
             ck.gemm_decode_grouped(ys, a, w2, offsets, 0, wr2, kc2, none, 1, t, 1)
-            kern.combine_sum(out, ys, pos, extra, k)
-            return out
+            return finish(ys, pos)
     if n <= MOE_BMM_MAX_ROWS or torch.cuda.is_current_stream_capturing():
         kern.gather_scaled(xs, x, None, w, k)
         sel = ids.reshape(-1).long()
         g = torch.bmm(w13.index_select(0, sel), xs.unsqueeze(2)).squeeze(2)
         ys = torch.bmm(w2.index_select(0, sel), gated_act(g, ACT_SILU).unsqueeze(2)).squeeze(2).contiguous()
-        kern.combine_sum(out, ys, None, extra, k)
-        return out
+        return finish(ys, None)
     offsets = torch.empty(e + 1, dtype=torch.int32, device=x.device)
     sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
     pos = torch.empty(n, dtype=torch.int32, device=x.device)
@@ -184,8 +199,7 @@ def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: to
         a0, a1 = off[ei], off[ei + 1]
         if a1 > a0:
             F.linear(gated_act(F.linear(xs[a0:a1], w13[ei]), ACT_SILU), w2[ei], out=ys[a0:a1])
-    kern.combine_sum(out, ys, pos, extra, k)
-    return out
+    return finish(ys, pos)
 
 
 def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
@@ -203,6 +217,20 @@ def latent_kv_write(cache: torch.Tensor, kv: torch.Tensor, w: torch.Tensor, posi
         ref.latent_kv_write(cache, kv, w, positions, slots, rank, rot_dim, inv_freq, eps)
         return
     _kern().latent_kv_write(cache, kv, w, positions, slots, rank, rot_dim, inv_freq, eps)
+
+
+def latent_qkv_prep(p: torch.Tensor, q_rank: int, wq: torch.Tensor, wkv: torch.Tensor, cache: torch.Tensor,
+                    positions: torch.Tensor, slots: torch.Tensor, rank: int, rot_dim: int, inv_freq: torch.Tensor,
+                    eps: float) -> torch.Tensor:
+    """Both consumers of the fused down-projection p [T, q_rank + rank + rot_dim] in one launch: returns
+    cq = rmsnorm(p[:, :q_rank]) * wq (model dtype) and writes the cache rows from p[:, q_rank:] as
+    :func:`latent_kv_write` does."""
+    if not p.is_cuda:
+        latent_kv_write(cache, p[:, q_rank:], wkv, positions, slots, rank, rot_dim, inv_freq, eps)
+        return rms_norm_ext(p[:, :q_rank], wq, eps)
+    cq = torch.empty(p.shape[0], q_rank, dtype=p.dtype, device=p.device)
+    _kern().latent_qkv_prep(cq, cache, p, wq, wkv, positions, slots, rank, rot_dim, inv_freq, eps)
+    return cq
 
 
 def latent_attn(q_lat: torch.Tensor, q: torch.Tensor, rot_off: int, cache: torch.Tensor, block_tables: torch.Tensor,

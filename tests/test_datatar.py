@@ -584,3 +584,45 @@ def test_generation_with_decode_graphs_and_decode_gemms(tmp_path):
     got = replay(eng, cut("z", prompts[1] + outs[1], [len(prompts[1])]))["z"]
     check_against_oracle(got, wts, cfg, prompts[1] + outs[1], TOL[torch.bfloat16])
     assert eng.blocks.num_available() == eng.blocks.num_blocks
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_launches_equal_their_parts(device, dtype):
+    """latent_qkv_prep = rms_norm_ext + latent_kv_write; moe_input_scaled(post_norm=...) = the expert sum followed
+    by post_norm_residual. On narrow (scalar path) and 8-aligned (16-byte path) widths."""
+    _need(device)
+    from src import ops
+
+    g = torch.Generator().manual_seed(7)
+    for q_rank, rank, rot in ((10, 12, 4), (16, 32, 16)):
+        t, bs = 9, 4
+        p = torch.randn(t, q_rank + rank + rot, generator=g).to(dtype).to(device)
+        wq = (1 + 0.1 * torch.randn(q_rank, generator=g)).to(dtype).to(device)
+        wkv = (1 + 0.1 * torch.randn(rank, generator=g)).to(dtype).to(device)
+        pos = torch.arange(3, 3 + t).to(device)
+        slots = torch.tensor([5, 0, -1, 7, 2, 11, 3, 9, 1]).to(device)
+        inv = ops.rope_inv_freq(100.0, rot, device)
+        c1 = torch.zeros(3, bs, rank + rot, dtype=dtype, device=device)
+        c2 = torch.zeros_like(c1)
+        cq = ops.latent_qkv_prep(p, q_rank, wq, wkv, c1, pos, slots, rank, rot, inv, 1e-5)
+        ops.latent_kv_write(c2, p[:, q_rank:], wkv, pos, slots, rank, rot, inv, 1e-5)
+        assert torch.equal(c1, c2) and float(c1.float().abs().sum()) > 0
+        assert torch.equal(cq, ops.rms_norm_ext(p[:, :q_rank], wq, 1e-5))
+    for h, f, tokens in ((12, 6, 5), (16, 8, 70)):
+        e, k = 4, 2
+        x = torch.randn(tokens, h, generator=g).to(dtype).to(device)
+        w13 = (torch.randn(e, 2 * f, h, generator=g) * 0.3).to(dtype).to(device)
+        w2 = (torch.randn(e, h, f, generator=g) * 0.3).to(dtype).to(device)
+        router = torch.randn(e, h, generator=g).to(dtype).to(device)
+        extra = torch.randn(tokens, h, generator=g).to(dtype).to(device)
+        nw = (0.2 * torch.randn(h, generator=g)).to(dtype).to(device)
+        w, ids = ops.route_sigmoid_topk(x, router, k)
+        r0 = torch.randn(tokens, h, generator=g).to(device)
+        want = r0.clone()
+        ops.post_norm_residual(want, ops.moe_input_scaled(x, w13, w2, w, ids, extra=extra), nw, 1e-5, True)
+        got = r0.clone()
+        act = torch.empty(tokens, h, dtype=torch.bfloat16, device=device)
+        assert ops.moe_input_scaled(x, w13, w2, w, ids, extra=extra, post_norm=(got, nw, 1e-5, True, act)) is None
+        assert (got - want).abs().max() < 1e-5 * want.abs().max()
+        assert torch.equal(act, got.to(torch.bfloat16))
