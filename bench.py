@@ -458,7 +458,7 @@ class _Watchdog:
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     args = parse(argv)
-    if args.design_compare:  # a separate measurement; the default workload and its JSON contract are untouched
+    if args.design_compare:  # a separate measurement; the default workload and its result line are untouched
         import importlib.util
         import shlex
 
