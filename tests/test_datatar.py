@@ -626,3 +626,50 @@ def test_fused_launches_equal_their_parts(device, dtype):
         assert ops.moe_input_scaled(x, w13, w2, w, ids, extra=extra, post_norm=(got, nw, 1e-5, True, act)) is None
         assert (got - want).abs().max() < 1e-5 * want.abs().max()
         assert torch.equal(act, got.to(torch.bfloat16))
+
+
+def test_worker_serves_a_datatar_checkpoint(tmp_path):
+    """The serving path end to end on the CPU: client -> coordinator -> worker -> LLMBackend -> from_pretrained
+    (the registry picks DatatarLM from config.json) -> continuous-batching engine -> sampled token ids, which are
+    the oracle's greedy continuation of each prompt."""
+    import asyncio
+
+    from src.client import InferenceClient
+    from src.config import ModelConfig
+    from src.coordinator import Coordinator
+    from src.worker import Worker
+
+    cfg = orc.make_config([(orc.mixer_cfg(), orc.dense_cfg()), (orc.mixer_cfg(heads=2, window=6), orc.dense_cfg(ff=16))],
+                          vocab=300, width=16)
+    wts = orc.make_weights(cfg, seed=22, dtype=torch.float32)
+    path = str(tmp_path / "served")
+    save_checkpoint(path, cfg, wts)
+    mc = ModelConfig(model_name="dt", model_path=path, arch="llama", max_batch_size=4, max_model_len=128,
+                     max_num_batched_tokens=128, num_kv_blocks=64, use_cuda_graph=False, max_latency_ms=1.0,
+                     overrides={"device": "cpu"})
+
+    async def main():
+        w = Worker("w0", host="127.0.0.1", install_signal_handlers=False)
+        assert w.load_model(mc)
+        wport = await w.start()
+        coord = Coordinator(port=0, max_batch_size=4, max_latency_ms=2)
+        cport = await coord.start()
+        await coord.add_static_worker(f"127.0.0.1:{wport}")
+        c = InferenceClient(f"127.0.0.1:{cport}")
+        prompts = [tokens_for(cfg, n, 40 + n) for n in (4, 19, 11)]
+        rs = await asyncio.wait_for(asyncio.gather(*(c.infer("dt", {"prompt_token_ids": p, "max_tokens": 6,
+                                                                    "ignore_eos": True}) for p in prompts)), 120)
+        c.close()
+        await coord.stop()
+        await w.shutdown()
+        return prompts, rs
+
+    prompts, rs = asyncio.run(main())
+    assert all(r["success"] for r in rs), rs
+    for p, r in zip(prompts, rs):
+        out = r["outputs"]["token_ids"]
+        assert len(out) == 6
+        lg = orc.forward(wts, cfg, p + out)
+        for i, tok in enumerate(out):
+            row = lg[len(p) + i - 1]
+            assert float(row.max() - row[tok]) <= 0.05 * float(row.max() - row.min())
