@@ -3,8 +3,8 @@
 // all heads of a token score against the SAME cached row [latent | rotated shared key part] and the output
 // is the weighted sum of the latent rows (W_uv is applied afterwards). One kernel serves prompt chunks and
 // single decode tokens: a row is a (token, head) pair, its keys are the cache positions j <= p inside the
-// sliding window, and the softmax denominator may hold a per-head sink term exp(sink_h) that has no key
-// and no value (running max starts at the sink, running sum at 1).
+// sliding window, and the softmax denominator may hold a per-head sink term exp(sink_h) attached to no position
+// (running max starts at the sink, running sum at 1).
 //
 // Scores, softmax weights and the weighted sum are fp32 (FMA); storage of q / cache / out is bf16 or fp32.
 // Workgroup = 4 waves x 4 rows. A tile of BK keys is staged once in LDS as fp32 (row stride odd: a lane per

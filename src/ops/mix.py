@@ -1,7 +1,7 @@
 """
 Dtype-generic ops (bf16 or fp32 storage, fp32 arithmetic) on the ``src/_Cmix`` HIP extension:
 
-* :func:`rms_norm_ext`, :func:`post_norm_residual` — RMS norms with a plain or a stored-around-zero weight,
+* :func:`rms_norm_ext`, :func:`post_norm_residual` — RMS norms with a plain weight or a `1 + w` gain,
   the second one applied to a sublayer's OUTPUT and added into an fp32 residual stream;
 * :func:`gated_act` — SiLU-gated and clamped sigmoid-gated feed-forward activations;
 * :func:`route_sigmoid_topk`, :func:`moe_input_scaled` — sigmoid-scored top-k routing whose weight scales
@@ -58,7 +58,7 @@ def _kern():
 def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_offset: bool = False,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x / sqrt(mean(x^2) + eps) * g over the last dim of [rows, n] (any row stride); g = w, or 1 + w with
-    ``unit_offset`` (a weight stored around zero), or 1 without a weight."""
+    ``unit_offset`` (the stored weight is an offset from one), or 1 without a weight."""
     out_dtype = out_dtype or x.dtype
     if not x.is_cuda:
         return ref.rms_norm_ext(x, w, eps, unit_offset, out_dtype)

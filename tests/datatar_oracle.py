@@ -27,7 +27,7 @@ def norm_plain(x, w, eps):
 
 
 def norm_around_zero(x, w, eps):
-    """weight stored around zero: the gain is 1 + w."""
+    """the stored weight is an offset from one: the gain is 1 + w."""
     return rms(x, eps) * (1.0 + w)
 
 
@@ -56,7 +56,8 @@ def window_mask(t: int, size: int) -> torch.Tensor:
 
 
 def softmax_with_sink(scores: torch.Tensor, ok: torch.Tensor, sink: Optional[torch.Tensor]) -> torch.Tensor:
-    """scores [H, T, T]; the denominator also holds exp(sink_h) once (no key, no value, not scaled)."""
+    """scores [H, T, T]; the denominator has one extra term exp(sink_h) per head, attached to no position and
+    left out of the score scaling."""
     e = torch.where(ok[None], torch.exp(scores - scores.masked_fill(~ok[None], -1e300).amax(-1, keepdim=True)), 0.0)
     # redo with an explicit common shift so that the sink enters on the same scale
     shift = scores.masked_fill(~ok[None], -1e300).amax(-1, keepdim=True)
