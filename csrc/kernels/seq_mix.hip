@@ -1,0 +1,509 @@
+// Kernels for models that carry per-sequence state besides the paged KV cache (gfx950). Storage of activations
+// is bf16 or fp32 (a run-time flag), arithmetic is fp32; recurrent state, residual streams, decays, gates of the
+// recurrence and unit norms are fp32 in both modes.
+//
+//   embed_hash          token embedding * scale + hashed bigram embedding -> S equal fp32 residual streams
+//   store_last_token    the step's last token of every sequence -> state (the next step's "previous token")
+//   stream_mix_norm     streams <- mix^T streams + out * y, and the next sublayer's input rmsnorm(in . streams) * g
+//   poly_norm_act       c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3
+//   delta_prep          short conv + SiLU of q/k/v, unit q/k, beta and decay of the gated delta rule
+//   conv_state_update   the convolution's trailing inputs -> state
+//   gated_delta         the recurrence itself, one workgroup per (sequence, head), state columns in registers
+//   qkv_prep            q/k norm, rotate-half rotary, value norm / value mixing, paged cache write
+#include "common.h"
+#include "seq_launchers.h"
+
+namespace die {
+
+namespace {
+
+__device__ __forceinline__ float ldv(const void* p, int64_t i, bool f32) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ void stv(void* p, int64_t i, bool f32, float v) {
+  if (f32)
+    reinterpret_cast<float*>(p)[i] = v;
+  else
+    reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
+}
+// the value as the activation dtype would hold it
+__device__ __forceinline__ float rnd(float v, bool f32) { return f32 ? v : bf2f(f2bf(v)); }
+__device__ __forceinline__ float siluf(float z) { return z / (1.0f + expf(-z)); }
+
+constexpr int NT = 256;
+
+// sequence of a row: the largest s with cu_q[s] <= row (cu_q == nullptr: the row itself)
+__device__ __forceinline__ int seq_of_row(const int* cu_q, int num_seqs, int row) {
+  if (cu_q == nullptr) return row;
+  int lo = 0, hi = num_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu_q[mid] <= row)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  return lo;
+}
+
+__global__ void __launch_bounds__(NT) embed_hash_kernel(float* streams, int S, int W, const void* embed,
+                                                       const void* bigram, bool f32, const int64_t* ids,
+                                                       RaggedRows r, const int64_t* prev_tok, float scale,
+                                                       int64_t buckets, int64_t mul_prev, int64_t mul_cur) {
+  const int row = blockIdx.x;
+  const int64_t tok = ids[row];
+  int64_t brow = -1;
+  if (bigram != nullptr) {
+    const int64_t p = r.positions[row];
+    if (p <= 0) {
+      brow = buckets;
+    } else {
+      const int s = seq_of_row(r.cu_q, r.num_seqs, row);
+      const int first = r.cu_q ? r.cu_q[s] : s;
+      const int64_t prev = row > first ? ids[row - 1] : prev_tok[r.state_slots[s]];
+      brow = (prev * mul_prev + tok * mul_cur) % buckets;
+    }
+  }
+  float* out = streams + (int64_t)row * S * W;
+  for (int c = threadIdx.x; c < W; c += NT) {
+    float x = ldv(embed, tok * W + c, f32) * scale;
+    if (brow >= 0) x += ldv(bigram, brow * W + c, f32);
+    for (int s = 0; s < S; ++s) out[(int64_t)s * W + c] = x;
+  }
+}
+
+__global__ void store_last_token_kernel(int64_t* prev_tok, const int64_t* ids, RaggedRows r) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= r.num_seqs) return;
+  const int last = r.cu_q ? r.cu_q[s + 1] - 1 : s;
+  if (r.cu_q && last < r.cu_q[s]) return;
+  prev_tok[r.state_slots[s]] = ids[last];
+}
+
+constexpr int SMAX = 8;
+
+__global__ void __launch_bounds__(NT) stream_mix_norm_kernel(StreamMixArgs a) {
+  __shared__ float red[NT / 64];
+  __shared__ float sm[SMAX * SMAX + 2 * SMAX];
+  const int S = a.S, W = a.W;
+  float* mixw = sm;
+  float* outw = sm + SMAX * SMAX;
+  float* inw = outw + SMAX;
+  if (threadIdx.x < S * S) mixw[threadIdx.x] = a.mix ? a.mix[threadIdx.x] : (threadIdx.x / S == threadIdx.x % S);
+  if (threadIdx.x < S) {
+    outw[threadIdx.x] = a.outw ? a.outw[threadIdx.x] : 1.0f;
+    inw[threadIdx.x] = a.inw ? a.inw[threadIdx.x] : 1.0f;
+  }
+  __syncthreads();
+  const int64_t t = blockIdx.x;
+  float* xs = a.streams + t * S * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += NT) {
+    float x[SMAX];
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) x[s] = s < S ? xs[(int64_t)s * W + c] : 0.f;
+    float u = 0.f;
+    if (a.y1 != nullptr) {
+      float y = a.a1 * ldv(a.y1, t * a.ys1 + c, a.y_f32);
+      if (a.y2 != nullptr) y += a.a2 * ldv(a.y2, t * a.ys2 + c, a.y_f32);
+#pragma unroll
+      for (int to = 0; to < SMAX; ++to) {
+        if (to < S) {
+          float n = outw[to] * y;
+#pragma unroll
+          for (int s = 0; s < SMAX; ++s)
+            if (s < S) n += mixw[s * S + to] * x[s];
+          xs[(int64_t)to * W + c] = n;
+          u += inw[to] * n;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < SMAX; ++s)
+        if (s < S) u += inw[s] * x[s];
+    }
+    ss += u * u;
+  }
+  if (a.h == nullptr) return;
+  ss = block_sum<NT>(ss, red);
+  const float rs = a.gain[0] / sqrtf(ss / (float)W + a.eps);
+  for (int c = threadIdx.x; c < W; c += NT) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s)
+      if (s < S) u += inw[s] * xs[(int64_t)s * W + c];  // this thread's own writes
+    stv(a.h, t * W + c, a.h_f32, u * rs);
+  }
+}
+
+__global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void* z, int64_t zstride, bool f32,
+                                                          const float* coef, float eps, int n) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int c = threadIdx.x; c < n; c += NT) {
+    const float v = ldv(z, r * zstride + c, f32);
+    const float v2 = v * v;
+    s2 += v2;
+    s4 += v2 * v2;
+    s6 += v2 * v2 * v2;
+  }
+  s2 = block_sum<NT>(s2, red);
+  s4 = block_sum<NT>(s4, red);
+  s6 = block_sum<NT>(s6, red);
+  const float r1 = coef[0] / sqrtf(s2 / (float)n + eps), r2 = coef[1] / sqrtf(s4 / (float)n + eps),
+              r3 = coef[2] / sqrtf(s6 / (float)n + eps), c3 = coef[3];
+  for (int c = threadIdx.x; c < n; c += NT) {
+    const float v = ldv(z, r * zstride + c, f32);
+    stv(out, r * n + c, f32, v * r1 + v * v * r2 + v * v * v * r3 + c3);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ gated delta rule
+__global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg, const void* x, const void* b,
+                                                       const void* a, int64_t xstride, bool f32, const float* conv_w,
+                                                       const float* conv_state, const float* A_log,
+                                                       const float* dt_bias, DeltaShape sh, RaggedRows r) {
+  extern __shared__ float vals[];  // [C]
+  const int row = blockIdx.x;
+  const int s = seq_of_row(r.cu_q, r.num_seqs, row);
+  const int first = r.cu_q ? r.cu_q[s] : s;
+  const int i = row - first;
+  const int64_t p = r.positions[row];
+  const int C = sh.channels(), taps = sh.taps;
+  const float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      if (p - back < 0) continue;
+      const int src = i - back;
+      const float xv = src >= 0 ? ldv(x, (int64_t)(row - back) * xstride + c, f32) : st[(int64_t)(taps - 1 + src) * C + c];
+      acc += conv_w[(int64_t)c * taps + j] * xv;
+    }
+    vals[c] = rnd(siluf(rnd(acc, f32)), f32);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = sh.kv_heads, d = sh.dim;
+  for (int hh = wave; hh < 2 * G; hh += NT / 64) {
+    float* v = vals + hh * d;
+    float ss = 0.f;
+    for (int c = lane; c < d; c += 64) ss += v[c] * v[c];
+    ss = wave_sum(ss);
+    float sc = 1.0f / sqrtf(ss + 1e-6f);
+    if (hh < G) sc *= 1.0f / sqrtf((float)d);
+    for (int c = lane; c < d; c += 64) v[c] *= sc;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += NT) qkv32[(int64_t)row * C + c] = vals[c];
+  const int H = sh.heads;
+  for (int h = threadIdx.x; h < H; h += NT) {
+    const float bv = ldv(b, (int64_t)row * xstride + h, f32);
+    const float av = ldv(a, (int64_t)row * xstride + h, f32) + dt_bias[h];
+    const float sp = av > 20.f ? av : log1pf(expf(av));
+    bg[(int64_t)row * 2 * H + h] = 1.0f / (1.0f + expf(-bv));
+    bg[(int64_t)row * 2 * H + H + h] = expf(-expf(A_log[h]) * sp);
+  }
+}
+
+constexpr int TAPS_MAX = 16;
+
+__global__ void __launch_bounds__(NT) conv_state_update_kernel(float* conv_state, const void* x, int64_t xstride,
+                                                              bool f32, DeltaShape sh, RaggedRows r) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * NT + threadIdx.x;
+  const int C = sh.channels(), taps = sh.taps;
+  if (c >= C) return;
+  const int q0 = r.cu_q ? r.cu_q[s] : s;
+  const int L = r.cu_q ? r.cu_q[s + 1] - q0 : 1;
+  if (L <= 0) return;
+  const int64_t p0 = r.positions[q0];
+  float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
+  float old[TAPS_MAX];
+#pragma unroll
+  for (int k = 0; k < TAPS_MAX; ++k) old[k] = k < taps - 1 ? st[(int64_t)k * C + c] : 0.f;
+  for (int k = 0; k < taps - 1; ++k) {
+    const int idx = L - 1 - (taps - 2 - k);  // row of the step that lands in place k
+    float v = 0.f;
+    if (idx >= 0) {
+      v = ldv(x, (int64_t)(q0 + idx) * xstride + c, f32);
+    } else if (p0 + idx >= 0) {
+      const int ok = taps - 1 + idx;
+#pragma unroll
+      for (int m = 0; m < TAPS_MAX; ++m)
+        if (m == ok) v = old[m];
+    }
+    st[(int64_t)k * C + c] = v;
+  }
+}
+
+constexpr int TB = 16;  // tokens staged per trip
+
+template <int DM>
+__global__ void __launch_bounds__(256) gated_delta_kernel(void* out, const float* qkv32, const float* bg,
+                                                         const void* gate, int64_t gstride, bool f32,
+                                                         const float* norm_w, float eps, float* state, DeltaShape sh,
+                                                         RaggedRows r) {
+  extern __shared__ float sm[];
+  const int d = sh.dim, dv = sh.vdim, H = sh.heads, G = sh.kv_heads, C = sh.channels();
+  float* qs = sm;               // [TB][d]
+  float* ks = qs + TB * d;      // [TB][d]
+  float* vs = ks + TB * d;      // [TB][dv]
+  float* os = vs + TB * dv;     // [TB][dv]
+  float* bs = os + TB * dv;     // [TB] beta
+  float* gs = bs + TB;          // [TB] decay
+  const int h = blockIdx.x, s = blockIdx.y, j = threadIdx.x, nthr = blockDim.x;
+  const int kh = h / (H / G);
+  const int q0 = r.cu_q ? r.cu_q[s] : s;
+  const int L = r.cu_q ? r.cu_q[s + 1] - q0 : 1;
+  if (L <= 0) return;
+  const bool fresh = r.positions[q0] <= 0;
+  float* st = state + ((int64_t)r.state_slots[s] * H + h) * d * dv;
+  float S[DM];
+#pragma unroll
+  for (int i = 0; i < DM; ++i) S[i] = (!fresh && i < d && j < dv) ? st[(int64_t)i * dv + j] : 0.f;
+  const int lane = j & 63, wave = j >> 6, nwaves = nthr >> 6;
+  for (int t0 = 0; t0 < L; t0 += TB) {
+    const int nb = min(TB, L - t0);
+    __syncthreads();
+    for (int e = j; e < nb * d; e += nthr) {
+      const int tt = e / d, c = e % d;
+      const float* row = qkv32 + (int64_t)(q0 + t0 + tt) * C;
+      qs[tt * d + c] = row[kh * d + c];
+      ks[tt * d + c] = row[G * d + kh * d + c];
+    }
+    for (int e = j; e < nb * dv; e += nthr) {
+      const int tt = e / dv, c = e % dv;
+      vs[tt * dv + c] = qkv32[(int64_t)(q0 + t0 + tt) * C + 2 * G * d + h * dv + c];
+    }
+    if (j < nb) {
+      bs[j] = bg[(int64_t)(q0 + t0 + j) * 2 * H + h];
+      gs[j] = bg[(int64_t)(q0 + t0 + j) * 2 * H + H + h];
+    }
+    __syncthreads();
+    if (j < dv) {
+      for (int tt = 0; tt < nb; ++tt) {
+        const float g = gs[tt], beta = bs[tt];
+        const float* kt = ks + tt * d;
+        const float* qt = qs + tt * d;
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < DM; ++i) {
+          if (i < d) {
+            S[i] *= g;
+            dot += S[i] * kt[i];
+          }
+        }
+        const float u = beta * (vs[tt * dv + j] - dot);
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DM; ++i) {
+          if (i < d) {
+            S[i] += kt[i] * u;
+            o += S[i] * qt[i];
+          }
+        }
+        os[tt * dv + j] = o;
+      }
+    }
+    __syncthreads();
+    for (int tt = wave; tt < nb; tt += nwaves) {
+      float ss = 0.f;
+      for (int c = lane; c < dv; c += 64) ss += os[tt * dv + c] * os[tt * dv + c];
+      ss = wave_sum(ss);
+      const float rs = 1.0f / sqrtf(ss / (float)dv + eps);
+      const int64_t row = q0 + t0 + tt;
+      for (int c = lane; c < dv; c += 64) {
+        const float gt = ldv(gate, row * gstride + h * dv + c, f32);
+        stv(out, (row * H + h) * dv + c, f32, os[tt * dv + c] * rs * norm_w[c] * siluf(gt));
+      }
+    }
+  }
+  if (j < dv) {
+#pragma unroll
+    for (int i = 0; i < DM; ++i)
+      if (i < d) st[(int64_t)i * dv + j] = S[i];
+  }
+}
+
+// --------------------------------------------------------------------------------------------------- qkv prep
+__global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
+  extern __shared__ float sm[];
+  __shared__ float red[NT / 64];
+  const int H = a.heads, G = a.kv_heads, d = a.dim, dv = a.vdim;
+  const int nq = H * d, nk = G * d, nv = G * dv;
+  float* qv = sm;
+  float* kv = qv + nq;
+  float* vv = kv + nk;
+  const int64_t t = blockIdx.x;
+  const bool f32 = a.f32;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < nq; c += NT) {
+    const float x = ldv(a.q, t * a.xstride + c, f32);
+    qv[c] = x;
+    sq += x * x;
+  }
+  for (int c = threadIdx.x; c < nk; c += NT) {
+    const float x = ldv(a.k, t * a.xstride + c, f32);
+    kv[c] = x;
+    sk += x * x;
+  }
+  float lam = 0.f;
+  if (a.v_lambda != nullptr) lam = a.v_lambda[0];
+  for (int c = threadIdx.x; c < nv; c += NT) {
+    float x = ldv(a.v, t * a.xstride + c, f32);
+    if (a.v_lambda != nullptr) x = (1.0f - lam) * x + lam * ldv(a.v_first, t * a.vfstride + c, f32);
+    vv[c] = x;
+  }
+  if (a.q_norm != nullptr) {
+    sq = block_sum<NT>(sq, red);
+    sk = block_sum<NT>(sk, red);
+    const float rq = 1.0f / sqrtf(sq / (float)nq + a.eps), rk = 1.0f / sqrtf(sk / (float)nk + a.eps);
+    for (int c = threadIdx.x; c < nq; c += NT) qv[c] *= rq * a.q_norm[c];
+    for (int c = threadIdx.x; c < nk; c += NT) kv[c] *= rk * a.k_norm[c];
+  }
+  __syncthreads();
+  if (a.rot_dims > 0) {
+    const int half = a.rot_dims / 2;
+    const float p = (float)a.positions[t];
+    for (int e = threadIdx.x; e < (H + G) * half; e += NT) {
+      const int hd = e / half, i = e % half;
+      float* base = hd < H ? qv + hd * d : kv + (hd - H) * d;
+      float sn, cs;
+      sincosf(p * a.inv_freq[i], &sn, &cs);
+      const float u = base[i], v = base[i + half];
+      base[i] = u * cs - v * sn;
+      base[i + half] = v * cs + u * sn;
+    }
+  }
+  if (a.v_unit) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int g = wave; g < G; g += NT / 64) {
+      float ss = 0.f;
+      for (int c = lane; c < dv; c += 64) ss += vv[g * dv + c] * vv[g * dv + c];
+      ss = wave_sum(ss);
+      const float rs = 1.0f / sqrtf(ss / (float)dv + a.eps);
+      for (int c = lane; c < dv; c += 64) vv[g * dv + c] *= rs;
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < nq; c += NT) stv(a.q_out, t * nq + c, f32, qv[c]);
+  const int64_t slot = a.slots[t];
+  if (slot < 0) return;
+  const int64_t dst = slot * (int64_t)(nk + nv);
+  for (int c = threadIdx.x; c < nk + nv; c += NT) stv(a.cache, dst + c, f32, kv[c]);  // kv and vv are adjacent
+}
+
+bool rows_ok(const RaggedRows& r) { return r.positions != nullptr && r.state_slots != nullptr && r.num_seqs >= 0; }
+
+}  // namespace
+
+hipError_t launch_embed_hash(float* streams, int S, int W, const void* embed, const void* bigram, bool f32,
+                             const int64_t* ids, RaggedRows r, const int64_t* prev_tok, float scale, int64_t buckets,
+                             int64_t mul_prev, int64_t mul_cur, hipStream_t s) {
+  if (r.total_rows == 0) return hipSuccess;
+  if (S < 1 || W < 1 || (bigram != nullptr && (buckets < 1 || prev_tok == nullptr || !rows_ok(r))))
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(embed_hash_kernel, dim3(r.total_rows), dim3(NT), 0, s, streams, S, W, embed, bigram, f32, ids, r,
+                     prev_tok, scale, buckets, mul_prev, mul_cur);
+  return hipGetLastError();
+}
+
+hipError_t launch_store_last_token(int64_t* prev_tok, const int64_t* ids, RaggedRows r, hipStream_t s) {
+  if (r.num_seqs == 0) return hipSuccess;
+  if (!rows_ok(r)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(store_last_token_kernel, dim3((r.num_seqs + 63) / 64), dim3(64), 0, s, prev_tok, ids, r);
+  return hipGetLastError();
+}
+
+hipError_t launch_stream_mix_norm(const StreamMixArgs& a, hipStream_t s) {
+  if (a.T == 0) return hipSuccess;
+  if (a.S < 1 || a.S > SMAX || a.W < 1 || (a.h != nullptr && a.gain == nullptr)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(stream_mix_norm_kernel, dim3(a.T), dim3(NT), 0, s, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_poly_norm_act(void* out, const void* z, int64_t zstride, bool f32, const float* coef, float eps,
+                                int rows, int n, hipStream_t s) {
+  if (rows == 0) return hipSuccess;
+  if (n < 1) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(poly_norm_act_kernel, dim3(rows), dim3(NT), 0, s, out, z, zstride, f32, coef, eps, n);
+  return hipGetLastError();
+}
+
+static bool delta_ok(const DeltaShape& sh) {
+  return sh.heads >= 1 && sh.kv_heads >= 1 && sh.heads % sh.kv_heads == 0 && sh.dim >= 1 && sh.dim <= 256 &&
+         sh.vdim >= 1 && sh.vdim <= 256 && sh.taps >= 1 && sh.taps <= TAPS_MAX;
+}
+
+hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void* b, const void* a, int64_t xstride,
+                             bool f32, const float* conv_w, const float* conv_state, const float* A_log,
+                             const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s) {
+  if (r.total_rows == 0) return hipSuccess;
+  if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
+  const size_t lds = sizeof(float) * sh.channels();
+  if (lds > 150 * 1024) return hipErrorInvalidValue;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(delta_prep_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(r.total_rows), dim3(NT), lds, s, qkv32, bg, x, b, a, xstride, f32, conv_w,
+                     conv_state, A_log, dt_bias, sh, r);
+  return hipGetLastError();
+}
+
+hipError_t launch_conv_state_update(float* conv_state, const void* x, int64_t xstride, bool f32, DeltaShape sh,
+                                    RaggedRows r, hipStream_t s) {
+  if (r.num_seqs == 0 || sh.taps <= 1) return hipSuccess;
+  if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(conv_state_update_kernel, dim3((sh.channels() + NT - 1) / NT, r.num_seqs), dim3(NT), 0, s,
+                     conv_state, x, xstride, f32, sh, r);
+  return hipGetLastError();
+}
+
+template <int DM>
+static hipError_t launch_gd(void* out, const float* qkv32, const float* bg, const void* gate, int64_t gstride, bool f32,
+                            const float* norm_w, float eps, float* state, DeltaShape sh, RaggedRows r, hipStream_t s) {
+  const int nthr = (sh.vdim + 63) / 64 * 64;
+  const size_t lds = sizeof(float) * (TB * (2 * sh.dim + 2 * sh.vdim) + 2 * TB);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gated_delta_kernel<DM>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(gated_delta_kernel<DM>, dim3(sh.heads, r.num_seqs), dim3(nthr), lds, s, out, qkv32, bg, gate,
+                     gstride, f32, norm_w, eps, state, sh, r);
+  return hipGetLastError();
+}
+
+hipError_t launch_gated_delta(void* out, const float* qkv32, const float* bg, const void* gate, int64_t gstride,
+                              bool f32, const float* norm_w, float eps, float* state, DeltaShape sh, RaggedRows r,
+                              hipStream_t s) {
+  if (r.num_seqs == 0 || r.total_rows == 0) return hipSuccess;
+  if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
+  if (sh.dim <= 32) return launch_gd<32>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  if (sh.dim <= 64) return launch_gd<64>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  if (sh.dim <= 128) return launch_gd<128>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  return launch_gd<256>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+}
+
+hipError_t launch_qkv_prep(const QkvPrepArgs& a, hipStream_t s) {
+  if (a.T == 0) return hipSuccess;
+  if (a.heads < 1 || a.kv_heads < 1 || a.heads % a.kv_heads != 0 || a.dim < 1 || a.vdim < 1 || a.rot_dims < 0 ||
+      a.rot_dims > a.dim || (a.rot_dims & 1) || (a.rot_dims > 0 && a.inv_freq == nullptr) ||
+      ((a.q_norm == nullptr) != (a.k_norm == nullptr)) || (a.v_lambda != nullptr && a.v_first == nullptr))
+    return hipErrorInvalidValue;
+  const size_t lds = sizeof(float) * ((size_t)a.heads * a.dim + (size_t)a.kv_heads * (a.dim + a.vdim));
+  if (lds > 150 * 1024) return hipErrorInvalidValue;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prep_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(qkv_prep_kernel, dim3(a.T), dim3(NT), lds, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace die

@@ -95,7 +95,8 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
     return out
 
 
-MIX_KERNELS = ["mix_ops", "latent_attn", "moe"]
+MIX_KERNELS = ["mix_ops", "latent_attn", "moe", "seq_mix", "sink_attn"]
+MIX_BINDINGS = ["bindings_mix", "bindings_seq"]
 # hipcc only: keeps -O3 from forming packed fp32 instructions out of ordinary float code
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -118,18 +119,19 @@ def build_mix(force: bool = False, jobs: int = 8, verbose: bool = False) -> str:
         if force or _newer(obj, [src] + hdrs + [os.path.abspath(__file__)]):
             jobs_list.append([HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", *NO_PACKED_FP32, "-I",
                               CSRC, "-c", src, "-o", obj])
-    bsrc = os.path.join(CSRC, "bindings_mix.cpp")
-    bobj = os.path.join(odir, "bindings_mix.o")
-    objs.append(bobj)
-    if force or _newer(bobj, [bsrc] + hdrs):
-        cmd = ["g++", "-O2", "-std=c++17", "-fPIC",
-               f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1",
-               "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_Cmix", "-DTORCH_API_INCLUDE_EXTENSION_H",
-               "-I", CSRC, "-I", "/opt/rocm/include", "-I", sysconfig.get_paths()["include"]]
-        for i in incs:
-            cmd += ["-isystem", i]
-        cmd += ["-c", bsrc, "-o", bobj]
-        jobs_list.append(cmd)
+    for b in MIX_BINDINGS:
+        bsrc = os.path.join(CSRC, b + ".cpp")
+        bobj = os.path.join(odir, b + ".o")
+        objs.append(bobj)
+        if force or _newer(bobj, [bsrc] + hdrs):
+            cmd = ["g++", "-O2", "-std=c++17", "-fPIC",
+                   f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1",
+                   "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_Cmix", "-DTORCH_API_INCLUDE_EXTENSION_H",
+                   "-I", CSRC, "-I", "/opt/rocm/include", "-I", sysconfig.get_paths()["include"]]
+            for i in incs:
+                cmd += ["-isystem", i]
+            cmd += ["-c", bsrc, "-o", bobj]
+            jobs_list.append(cmd)
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         for res in ex.map(_run, jobs_list):
             if verbose and res:

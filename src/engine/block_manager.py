@@ -39,7 +39,12 @@ def native_runtime():
 
 class KVBlockManager:
     def __init__(self, num_blocks: int, block_size: int, enable_prefix_caching: bool = True,
-                 ttl_s: Optional[float] = None, salt: int = 0):
+                 ttl_s: Optional[float] = None, salt: int = 0, state_slots: int = 0):
+        # state slots (models with per-sequence state besides the cache): a sequence takes one with its first
+        # blocks and gives it back with them, so admission, preemption, abort and finish all keep the two in step;
+        # the lowest free slot is handed out first
+        self._free_slots: List[int] = list(range(state_slots))
+        self.num_state_slots = state_slots
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.prefix_caching = enable_prefix_caching
@@ -58,6 +63,18 @@ class KVBlockManager:
         return self.bm.num_used() / self.num_blocks
 
     # -------------------------------------------------------- allocation
+    def _take_state_slot(self, seq: Sequence) -> None:
+        if self.num_state_slots and seq.state_slot is None:
+            if not self._free_slots:
+                raise RuntimeError("no free state slot: more live sequences than the state pool holds")
+            self._free_slots.sort()
+            seq.state_slot = self._free_slots.pop(0)
+
+    def _drop_state_slot(self, seq: Sequence) -> None:
+        if seq.state_slot is not None:
+            self._free_slots.append(seq.state_slot)
+            seq.state_slot = None
+
     def _prompt_hashes(self, seq: Sequence) -> List[int]:
         if seq.block_hashes is None:
             seq.block_hashes = list(self._hash(seq.prompt_ids, self.block_size, 0, self.salt))
@@ -84,6 +101,7 @@ class KVBlockManager:
                 self.bm.free(matched)
             raise
         seq.block_table = matched + fresh
+        self._take_state_slot(seq)
         seq.num_computed = len(matched) * self.block_size
         seq.num_prefix_hit = seq.num_computed
 
@@ -91,6 +109,7 @@ class KVBlockManager:
         """A table of ``n_blocks`` new blocks (no prefix matching): swap-in target."""
         assert not seq.block_table
         seq.block_table = list(self.bm.allocate(n_blocks))
+        self._take_state_slot(seq)
         return list(seq.block_table)
 
     def ensure_slots(self, seq: Sequence, n_tokens: int) -> bool:
@@ -101,6 +120,7 @@ class KVBlockManager:
         if need > self.bm.num_available():
             return False
         seq.block_table.extend(self.bm.allocate(need))
+        self._take_state_slot(seq)
         return True
 
     def register_prompt_blocks(self, seq: Sequence) -> None:
@@ -116,6 +136,7 @@ class KVBlockManager:
         if seq.block_table:
             self.bm.free(seq.block_table)
         seq.block_table = []
+        self._drop_state_slot(seq)
 
     def evict_expired(self) -> int:
         return self.bm.evict_expired()

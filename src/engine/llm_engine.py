@@ -115,7 +115,16 @@ class LLMEngine:
                                self.device, dtype=model.dtype)
             per_block = KVPool.bytes_per_block(self.arch.num_layers, model.hkv, cfg.block_size, self.arch.head_dim)
             can_move = True
-        self.blocks = KVBlockManager(nblocks, cfg.block_size, cfg.enable_prefix_caching, cfg.kv_block_ttl_s)
+        prefix = cfg.enable_prefix_caching and getattr(model, "supports_prefix_cache", True)
+        n_state = 0
+        if getattr(model, "needs_seq_state", False):
+            # per-sequence state besides the cache (recurrent layers, the previous token): one slot per live
+            # sequence, handed out and taken back with the sequence's cache blocks. Such state is not part of
+            # the block movers' packets, so these models recompute on preemption and keep no prefix cache
+            n_state = cfg.max_num_seqs
+            self.seq_state = model.make_seq_state(n_state)
+            can_move = False
+        self.blocks = KVBlockManager(nblocks, cfg.block_size, prefix, cfg.kv_block_ttl_s, state_slots=n_state)
         self.runner = runner_cls(model, self.pool, cfg, self.max_model_len)
         # host swap space for preempted sequences (single-process runners only: a TP group would
         # have to mirror every swap on its followers, so it always recomputes)
@@ -213,6 +222,9 @@ class LLMEngine:
 
     def _add_imported(self, packet, sampling: SamplingParams, on_finish) -> Sequence:
         from src.parallel.kv_transfer import import_blocks
+
+        if getattr(self.model, "needs_seq_state", False):
+            raise ValueError("a model with per-sequence state cannot resume from shipped KV blocks alone")
 
         if packet.block_size != self.cfg.block_size:
             raise ValueError("block size mismatch between prefill and decode workers")

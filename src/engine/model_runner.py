@@ -86,6 +86,11 @@ class ModelRunner:
         self.h_ctx = torch.zeros(self.max_seqs, dtype=i32, pin_memory=pin)
         self.h_bt = torch.zeros(self.max_seqs, self.bt_width, dtype=i32, pin_memory=pin)
         self.h_last = torch.zeros(self.max_seqs, dtype=i64, pin_memory=pin)
+        # state slot per sequence of the step (models with per-sequence state; rows past the real ones keep the
+        # pool's spare slot)
+        self.uses_state = bool(getattr(model, "needs_seq_state", False))
+        self.pad_state_slot = model.seq_state.pad_slot if self.uses_state and model.seq_state is not None else 0
+        self.h_sslot = torch.full((self.max_seqs,), self.pad_state_slot, dtype=i32, pin_memory=pin)
         self.h_temp = torch.zeros(self.max_seqs, dtype=torch.float32, pin_memory=pin)
         self.h_topk = torch.zeros(self.max_seqs, dtype=i32, pin_memory=pin)
         self.h_topp = torch.ones(self.max_seqs, dtype=torch.float32, pin_memory=pin)
@@ -118,6 +123,7 @@ class ModelRunner:
         self.d_ctx = torch.ones(self.max_seqs, dtype=i32, device=dev)
         self.d_bt = torch.zeros(self.max_seqs, self.bt_width, dtype=i32, device=dev)
         self.d_last = torch.zeros(self.max_seqs, dtype=i64, device=dev)
+        self.d_sslot = torch.full((self.max_seqs,), self.pad_state_slot, dtype=i32, device=dev)
         self.d_temp = torch.zeros(self.max_seqs, dtype=torch.float32, device=dev)
         self.d_topk = torch.zeros(self.max_seqs, dtype=i32, device=dev)
         self.d_topp = torch.ones(self.max_seqs, dtype=torch.float32, device=dev)
@@ -165,6 +171,19 @@ class ModelRunner:
         if with_cu:
             self.d_cu[: n_seq + 1].copy_(self.h_cu[: n_seq + 1], non_blocking=nb)
             self.d_last[:n_seq].copy_(self.h_last[:n_seq], non_blocking=nb)
+        if self.uses_state:
+            self.d_sslot[:n_seq].copy_(self.h_sslot[:n_seq], non_blocking=nb)
+
+    def _stage_state_slots(self, seqs: Seq[Sequence], n_pad: int) -> None:
+        if not self.uses_state:
+            return
+        ns = self.h_sslot.numpy()
+        n = len(seqs)
+        ns[:n] = [s.state_slot for s in seqs]
+        ns[n:n_pad] = self.pad_state_slot
+
+    def _state_slots(self, n: int) -> Optional[torch.Tensor]:
+        return self.d_sslot[:n] if self.uses_state else None
 
     def _fill_sampling(self, seqs: Seq[Sequence], n_pad: int) -> bool:
         """Write per-row sampling params; returns True when every row is greedy.
@@ -244,6 +263,7 @@ class ModelRunner:
         (None for partial prompt chunks)."""
         n = len(chunks)
         t = self._stage_chunks(chunks)
+        self._stage_state_slots([c.seq for c in chunks], n)
         done = [i for i, c in enumerate(chunks) if c.completes_prompt]
         nd = len(done)
         if nd and nd != n:
@@ -282,17 +302,18 @@ class ModelRunner:
         chunk tokens). A batch of single tokens runs the decode form of the step (one query row per sequence)."""
         n = len(chunks)
         t = self._stage_chunks(chunks)
+        self._stage_state_slots([c.seq for c in chunks], n)
         self._h2d(t, n, with_cu=True)
         dev = self.device
         single = all(c.length == 1 for c in chunks)
         if single:
             meta = AttnMetadata(is_prefill=False, slot_mapping=self.d_slots[:n], block_tables=self.d_bt[:n],
                                 ctx_lens=self.d_ctx[:n], max_ctx=self.max_model_len, part_o=self.part_o,
-                                part_ml=self.part_ml, attn_cnt=self.attn_cnt)
+                                part_ml=self.part_ml, attn_cnt=self.attn_cnt, state_slots=self._state_slots(n))
         else:
             meta = AttnMetadata(is_prefill=True, slot_mapping=self.d_slots[:t], block_tables=self.d_bt[:n],
                                 ctx_lens=self.d_ctx[:n], cu_q=self.d_cu[: n + 1],
-                                max_q_len=max(c.length for c in chunks))
+                                max_q_len=max(c.length for c in chunks), state_slots=self._state_slots(n))
         hidden = self.model.forward(self.d_ids[:t], self.d_pos[:t], meta, self.pool.tensor)
         if not rows:
             if self.is_cuda:
@@ -307,7 +328,7 @@ class ModelRunner:
         keep = self.d_last[:nd] if self.prune_last else None
         meta = AttnMetadata(is_prefill=True, slot_mapping=self.d_slots[:t], block_tables=self.d_bt[:n],
                             ctx_lens=self.d_ctx[:n], cu_q=self.d_cu[: n + 1], max_q_len=max_q, kv_hook=kv_hook,
-                            keep_rows=keep)
+                            keep_rows=keep, state_slots=self._state_slots(n))
         hidden = self.model.forward(self.d_ids[:t], self.d_pos[:t], meta, self.pool.tensor)
         if not nd:
             return None
@@ -335,7 +356,7 @@ class ModelRunner:
         meta = AttnMetadata(is_prefill=False, slot_mapping=self.d_slots[:n], block_tables=self.d_bt[:n],
                             ctx_lens=self.d_ctx[:n], max_ctx=self.max_model_len, part_o=self.part_o,
                             part_ml=self.part_ml, attn_cnt=self.attn_cnt, scratch=self.dec_scratch,
-                            pre_embedded=tail)
+                            pre_embedded=tail, state_slots=self._state_slots(n))
         hidden = self.model.forward(self.d_ids[:n], self.d_pos[:n], meta, self.pool.tensor)
         amax = (self.d_lmpart if self.d_lmpart is not None and n <= ops.DECODE_GEMM_MAX_M
                 and self.model.lm_head_argmax_parts() == self.d_lmpart.shape[1] else None)
@@ -399,6 +420,7 @@ class ModelRunner:
                                     self.h_pos.data_ptr(), self.h_slots.data_ptr(), self.h_ctx.data_ptr(),
                                     self.h_bt.data_ptr(), self.bt_width, pad)
         self._fill_sampling(seqs, pad)
+        self._stage_state_slots(seqs, pad)
         self._h2d(pad, pad, with_cu=False)
         self._pre_embed(pad)  # the step starts from these rows when its tail launch writes the next ones
         if self.supports_multistep:  # the graph's input advance must see this step's real rows
@@ -433,6 +455,7 @@ class ModelRunner:
                                     self.h_pos.data_ptr(), self.h_slots.data_ptr(), self.h_ctx.data_ptr(),
                                     self.h_bt.data_ptr(), self.bt_width, pad)
         self._fill_sampling(seqs, pad)
+        self._stage_state_slots(seqs, pad)
         self._h2d(pad, pad, with_cu=False)
         self._pre_embed(pad)  # the step starts from these rows when its tail launch writes the next ones
         self.h_ctl[0] = 0

@@ -43,6 +43,7 @@ class Sequence:
     # Disaggregation: a sequence whose prompt KV arrives from a prefill worker
     imported_kv: bool = False
     swap_buf: Any = None             # host copy of the KV blocks while SWAPPED
+    state_slot: Optional[int] = None  # slot in the model's per-sequence state pool while it holds cache blocks
 
     def __len__(self) -> int:
         return len(self.prompt_ids) + len(self.output_ids)

@@ -56,6 +56,9 @@ class AttnMetadata:
     # decode (fused path): the step's embedding rows and first-norm statistics are already in scratch["h_in"] /
     # scratch["ssp0"] (written by the previous step's sampling launch, or by the runner before a window)
     pre_embedded: bool = False
+    # models with per-sequence state besides the cache (recurrent layers, the previous token): the state slot of
+    # every sequence of the step, [S] int32 (padded rows of a captured decode step: the pool's spare slot)
+    state_slots: Optional[torch.Tensor] = None
 
 
 class LayerWeights:

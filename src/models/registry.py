@@ -2,7 +2,9 @@
 Model-class registry: which model class serves a checkpoint directory, decided by its ``config.json``.
 
 * HuggingFace-format Llama / Mistral / Mixtral (``model_type``) -> :class:`src.models.llama.CausalLM`;
-* ``"architecture": "Datatar"`` (layers listed in the config) -> :class:`src.models.datatar.DatatarLM`.
+* ``"architecture": "Datatar"`` (layers listed in the config) -> :class:`src.models.datatar.DatatarLM`;
+* ``"architecture": "Fekolorn"`` (layers listed in the config, per-sequence state) ->
+  :class:`src.models.fekolorn.FekolornLM`.
 
 A new family registers a (matcher, arch reader, model class) triple with :func:`register_family`.
 """
@@ -73,6 +75,19 @@ def _datatar_arch(path: str, **kw):
     return datatar_arch_from_dir(path, **kw)
 
 
+def _fekolorn_cls():
+    from src.models.fekolorn import FekolornLM
+
+    return FekolornLM
+
+
+def _fekolorn_arch(path: str, **kw):
+    from src.models.fekolorn import fekolorn_arch_from_dir
+
+    return fekolorn_arch_from_dir(path, **kw)
+
+
 register_family("datatar", lambda c: c.get("architecture") == "Datatar", _datatar_arch, _datatar_cls)
+register_family("fekolorn", lambda c: c.get("architecture") == "Fekolorn", _fekolorn_arch, _fekolorn_cls)
 register_family("llama", lambda c: "architecture" not in c and c.get("model_type", "llama") in
                 ("llama", "mistral", "mixtral"), _llama_arch, _llama_cls)

@@ -60,10 +60,11 @@ def main(argv=None) -> int:
     from src.models.registry import family_of
 
     family = family_of(a.model)
-    if family != "datatar" and a.dtype == "float32":
+    generic = family in ("datatar", "fekolorn")   # families on the dtype-generic kernels (src/_Cmix) alone
+    if not generic and a.dtype == "float32":
         print(f"the {family} kernels are bfloat16 only", file=sys.stderr)
         return 3
-    _ensure_built(need_full=family != "datatar")
+    _ensure_built(need_full=not generic)
 
     import numpy as np
     import torch
