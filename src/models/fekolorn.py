@@ -25,6 +25,7 @@ from :class:`src.models.datatar.LayerRowPool`, state slots from :class:`SeqState
 from __future__ import annotations
 
 import json
+import math
 import os
 from dataclasses import dataclass, replace
 from typing import Any, Dict, List, Optional, Tuple
@@ -250,7 +251,9 @@ class SinkAttentionMixer:
         self.q_norm = (1.0 + rnd(self.nq, scale=0.1, dt=f32)) if s.qk_norm else None
         self.k_norm = (1.0 + rnd(self.nk, scale=0.1, dt=f32)) if s.qk_norm else None
         self.vmix = (0.3 + rnd(1, scale=0.05, dt=f32)) if s.v_mix else None
-        self.rel_rows = 32
+        # buckets of the distance bias: a checkpoint's tensor decides (load); a random model takes up to 32, half
+        # of them below bias_max
+        self.rel_rows = max(2, min(32, 2 * (math.ceil(s.bias_max) - 1)))
         self.rel = rnd(self.rel_rows, s.heads, scale=0.5, dt=f32) if s.bias_max else None
         self.bias = None
         self.inv_freq = mix.rope_inv_freq(s.rot_base, s.rot_dims, self.device) if s.rot_dims else None

@@ -61,6 +61,8 @@ def distance_bias_table(rel: torch.Tensor, bias_max: float, window: int = 0) -> 
     for n in range(top + 1):
         if n < half or half == 0:
             idx.append(min(n, B - 1))
+        elif bias_max <= half:   # no room for shared buckets: everything from B // 2 on takes the last one
+            idx.append(B - 1)
         else:
             idx.append(min(B - 1, half + int(math.floor(math.log(n / half) / math.log(bias_max / half) * (B - half)))))
     return rel.float()[torch.tensor(idx, device=rel.device)].contiguous()

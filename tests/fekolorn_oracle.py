@@ -21,10 +21,6 @@ def rms(x: torch.Tensor, eps: float) -> torch.Tensor:
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def silu(z: torch.Tensor) -> torch.Tensor:
     return z * torch.sigmoid(z)
 
@@ -222,3 +218,92 @@ def forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict, layer_out:
             layer_out.append(sum(xs))
     x = scalar_norm(sum(xs), w["final.norm"], eps)
     return x @ w["head"].T
+
+
+# --------------------------------------------------------------------------------- configurations and weights
+def attn_cfg(heads=4, kv_heads=2, dim=16, vdim=8, window=6, bias_max=10, v_mix=True, scale=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "bias_max": bias_max, "v_mix": v_mix,
+         "scale": scale if scale is not None else dim ** -0.5}
+    if window:
+        m["mask"] = {"size": window}
+    return m
+
+
+def parallel_cfg(heads=4, kv_heads=2, dim=16, vdim=8, rot_dims=8, rot_base=100.0, r_heads=2, r_kv_heads=1, r_dim=8,
+                 r_vdim=16, conv=3, left_scale=0.7, right_scale=1.1):
+    return {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                     "rot": {"base": rot_base, "dims": rot_dims}},
+            "right": {"heads": r_heads, "kv_heads": r_kv_heads, "dim": r_dim, "vdim": r_vdim, "conv": conv},
+            "left_scale": left_scale, "right_scale": right_scale}
+
+
+def make_config(layers, width=32, vocab=50, streams=2, buckets=37, eps=1e-5, embed_scale=0.7):
+    """layers: list of (type, mixer config, ff or None)."""
+    c = {"architecture": "Fekolorn", "embedding": {"scale": embed_scale}, "norm": {"eps": eps}, "vocab": vocab,
+         "width": width,
+         "layers": [{"type": t, "mixer": m, "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+                    for t, m, ff in layers]}
+    if buckets:
+        c["embedding"]["bigram"] = {"buckets": buckets, "mul_prev": 5, "mul_cur": 3}
+    if streams:
+        c["streams"] = streams
+    return c
+
+
+def make_weights(cfg: dict, seed: int = 0, rel_rows: int = 12) -> Dict[str, torch.Tensor]:
+    """Random tensors under the checkpoint's names, every value exactly representable in bfloat16."""
+    g = torch.Generator().manual_seed(seed)
+    W, S = cfg["width"], cfg.get("streams")
+    w: Dict[str, torch.Tensor] = {}
+
+    def r(*shape, std=1.0, mean=0.0):
+        return (torch.randn(shape or (1,), generator=g) * std + mean).bfloat16()
+
+    lin = lambda o, i: r(o, i, std=i ** -0.5)  # noqa: E731
+    w["embed"] = r(cfg["vocab"], W)
+    bg = cfg["embedding"].get("bigram")
+    if bg:
+        w["bigram"] = r(bg["buckets"] + 1, W, std=0.7)
+    for li, lc in enumerate(cfg["layers"]):
+        p = f"l{li}."
+        for q in (1, 2):
+            if q == 2 and lc["mlp"] is None:
+                continue
+            w[p + f"norm{q}"] = r(std=0.1, mean=1.0).reshape(())
+            if S:
+                w[p + f"hc{q}.in"] = r(S, std=0.2, mean=1.0 / S)
+                w[p + f"hc{q}.out"] = r(S, std=0.2, mean=0.8)
+                w[p + f"hc{q}.mix"] = (torch.eye(S) * 0.9 + torch.randn(S, S, generator=g) * 0.1).bfloat16()
+        m = lc["mixer"]
+
+        def attn(pre, a, biased):
+            H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            w[pre + "q"], w[pre + "k"], w[pre + "v"] = lin(H * d, W) * 2, lin(G * d, W) * 2, lin(G * dv, W)
+            w[pre + "o"] = lin(W, H * dv)
+            w[pre + "sink"] = r(H, std=1.0)
+            if biased:
+                w[pre + "q.norm"], w[pre + "k.norm"] = r(H * d, std=0.2, mean=1.5), r(G * d, std=0.2, mean=1.5)
+                w[pre + "rel"] = r(rel_rows, H, std=1.0)
+                w[pre + "vmix"] = r(std=0.1, mean=0.4).reshape(())
+
+        if lc["type"] == "attention":
+            attn(p + "mix.", m, True)
+        else:
+            attn(p + "mix.left.", m["left"], False)
+            a = m["right"]
+            H, G, d, dv, taps = a["heads"], a["kv_heads"], a["dim"], a["vdim"], a["conv"]
+            pre = p + "mix.right."
+            w[pre + "q"], w[pre + "k"], w[pre + "v"] = lin(G * d, W) * 2, lin(G * d, W) * 2, lin(H * dv, W) * 2
+            for nm, n in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                w[pre + nm + ".conv"] = r(n, taps, std=0.6)
+            w[pre + "b"], w[pre + "a"] = lin(H, W) * 2, lin(H, W) * 2
+            w[pre + "A_log"], w[pre + "dt_bias"] = r(H, std=0.5, mean=-0.5), r(H, std=0.5)
+            w[pre + "norm"] = r(dv, std=0.2, mean=1.0)
+            w[pre + "g"], w[pre + "o"] = lin(H * dv, W) * 2, lin(W, H * dv)
+        if lc["mlp"] is not None:
+            ff = lc["mlp"]["ff"]
+            w[p + "mlp.up"], w[p + "mlp.down"] = lin(ff, W) * 2, lin(W, ff)
+            w[p + "mlp.act"] = r(4, std=0.5, mean=0.3)
+    w["final.norm"] = r(std=0.1, mean=1.0).reshape(())
+    w["head"] = lin(cfg["vocab"], W)
+    return w
