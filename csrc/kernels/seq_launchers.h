@@ -117,6 +117,12 @@ struct SinkAttnArgs {
   float scale;
   bool f32;
   int impl;               // 0: matrix cores where they apply, else FMA; 1: FMA; 2: matrix cores or fail
+  // split keys (matrix-core kernel only): nsplit > 1 workgroups per row tile take `chunk` keys each and write
+  // unnormalised partial sums to ws_o [nsplit, T * H, vdim] and (running max in log2 units, sum) to
+  // ws_ml [nsplit, T * H, 2]; a merge kernel then writes `out`
+  float* ws_o;
+  float* ws_ml;
+  int nsplit, chunk;
 };
 hipError_t launch_sink_attn(const SinkAttnArgs& a, hipStream_t s);
 bool sink_attn_uses_mfma(const SinkAttnArgs& a);

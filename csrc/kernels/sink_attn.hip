@@ -9,7 +9,7 @@
 // FMA form (any shape, both storage types): a workgroup of 4 waves owns 4 * RPW rows (a row = one token and one
 // of the H / G query heads of ONE key/value head), stages tiles of BK keys and values once in LDS as fp32 (odd row
 // stride) and shares them between its rows. Lanes split (key, slice of dim) for the scores, value columns for the
-// weighted sum.
+// weighted sum. The matrix-core form for bf16 follows it below.
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -187,15 +187,306 @@ template <bool F32> hipError_t launch_fma(const SinkAttnArgs& a, hipStream_t s) 
   return launch_cc<64, 4, F32>(a, s);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// bf16 on the matrix cores (v_mfma_f32_32x32x16_bf16), for dim % 16 == 0, dim <= 128, vdim % 32 == 0, vdim <= 128.
+// Workgroup = NW waves x 32 rows of one (sequence, key/value head); NW = 1 for steps of few rows (decode). Per tile
+// of 32 keys, staged once in LDS as rows [K_g | V_g] (the next tile's global loads in flight meanwhile):
+//   S^T[key][q] = K Q^T        A = K rows from LDS, B = Q rows from LDS      (dim / 16 MFMAs)
+//   online softmax per query column (a lane pair owns a query), fp32 scores and weights in log2 units, the bias
+//   per distance added before, the running max seeded with the sink; P is rounded to bf16 only as MFMA operand
+//   O^T[d][q] += V^T P^T      A = the value columns of the same tile read transposed (ds_read_tr16_b64),
+//                              B = P^T straight from the score accumulator   (2 * vdim / 32 MFMAs)
+// Split keys (decode over long contexts): split z takes keys [jlo + z * chunk, + chunk) and writes its
+// unnormalised O, running max and sum to a workspace; sink_attn_merge_kernel combines them. The sink enters
+// split 0 only.
+constexpr int MKT = 32;
+constexpr int BT_LDS_MAX = 2048;
+typedef __attribute__((address_space(3))) short4_t lds_short4;
+typedef __attribute__((ext_vector_type(8))) short short8_t;
+
+template <int NDB, int NW, int NKC>
+__global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a, int KP, int QP, float* ws_o,
+                                                                float* ws_ml, int nsplit, int chunk) {
+  constexpr int ROWS = 32 * NW, NT = 64 * NW;
+  constexpr int NPF = (MKT * (4 * NDB + NKC) + NT - 1) / NT;  // 16-byte chunks of a key tile per thread
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [ROWS][QP]
+  bf16_t* ks = qs + ROWS * QP;                                // [MKT][KP] = [K_g | V_g]
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    // XCD k (workgroups are dealt round-robin by linear id) takes a contiguous eighth of the sequence-major tile
+    // list, so one sequence's cache rows stay in one L2
+    const unsigned total = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
+    if (total % 8 == 0) {
+      const unsigned nl = (lin % 8) * (total / 8) + lin / 8;
+      bx = (int)(nl % gridDim.x);
+      by = (int)(nl / gridDim.x);
+    }
+  }
+  const int H = a.heads, G = a.kv_heads, QPG = H / G, D = a.dim, DV = a.vdim;
+  const int s = by, g = blockIdx.z % G, z = blockIdx.z / G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  const int roww = G * (D + DV);
+  const int q0 = a.cu_q ? a.cu_q[s] : s;
+  const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
+  const int nrows = nq * QPG, row0 = bx * ROWS;
+  if (row0 >= nrows) return;
+  const int ctx = a.ctx_lens[s];
+  const int last_row = min(row0 + ROWS, nrows) - 1;
+  const int p_first = (int)a.positions[q0 + row0 / QPG], p_last = (int)a.positions[q0 + last_row / QPG];
+  int jlo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  int jhi = min(p_last, ctx - 1);
+  if (nsplit > 1) {
+    jlo += z * chunk;
+    jhi = min(jhi, jlo + chunk - 1);
+  }
+  const bf16_t* qg = reinterpret_cast<const bf16_t*>(a.q);
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+  const int qcol = lane & 31, hh = lane >> 5;
+  const int myrow = row0 + wave * 32 + qcol;
+  const bool rok = myrow < nrows;
+  const int myh = g * QPG + (rok ? myrow % QPG : 0);
+  const int64_t orow = rok ? (int64_t)(q0 + myrow / QPG) * H + myh : 0;
+  const int64_t wrows = (int64_t)a.total_q * H;
+  if (jlo > jhi) {  // an empty split (uniform over the workgroup): it only reports that it holds nothing
+    if (nsplit > 1 && rok && hh == 0) {
+      ws_ml[((int64_t)z * wrows + orow) * 2] = -1e30f;
+      ws_ml[((int64_t)z * wrows + orow) * 2 + 1] = 0.f;
+    }
+    return;
+  }
+
+  const int lch = D / 8;
+  for (int idx = tid; idx < ROWS * lch; idx += NT) {
+    const int r = idx / lch, c = idx % lch, row = row0 + r;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < nrows) {
+      const int64_t t = q0 + row / QPG;
+      v = *reinterpret_cast<const uint4*>(qg + (t * H + g * QPG + row % QPG) * D + 8 * c);
+    }
+    *reinterpret_cast<uint4*>(qs + r * QP + 8 * c) = v;
+  }
+
+  const bool wave_live = row0 + wave * 32 < nrows;
+  const int prow = rok ? (int)a.positions[q0 + myrow / QPG] : -1;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float sl2 = a.scale * LOG2E;
+  const bool has_sink = a.sink != nullptr && rok && z == 0;
+  float m = has_sink ? a.sink[myh] * LOG2E : -1e30f;
+  float l = has_sink ? 1.0f : 0.0f;
+  f32x16_t o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+
+  const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
+  const int kchK = D / 8, kch = (D + DV) / 8, nkk = D / 16, nchunks = MKT * kch;
+  int* btl = reinterpret_cast<int*>(ks + MKT * KP);
+  const int b_lo = jlo / a.block_size, nbt = jhi / a.block_size - b_lo + 1;
+  const bool bt_lds = nbt <= BT_LDS_MAX;
+  if (bt_lds)
+    for (int u = tid; u < nbt; u += NT) btl[u] = bt[b_lo + u];
+  uint4 pf[NPF];
+  auto fetch = [&](int j0, bool lds) {
+#pragma unroll
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      const int k = idx / kch, c = idx % kch, j = j0 + k;
+      pf[u] = make_uint4(0, 0, 0, 0);
+      if (idx < nchunks && j <= jhi) {
+        const int jb = j / a.block_size;
+        const int64_t blk = lds ? btl[jb - b_lo] : bt[jb];
+        const int64_t rowp = (blk * a.block_size + (j - jb * a.block_size)) * roww;
+        const int64_t col = c < kchK ? (int64_t)g * D + 8 * c : (int64_t)G * D + (int64_t)g * DV + 8 * (c - kchK);
+        pf[u] = *reinterpret_cast<const uint4*>(cache + rowp + col);
+      }
+    }
+  };
+  fetch(jlo, false);
+  const int pitchB = KP * 2;
+  const int g16 = lane >> 4, i16 = lane & 15;
+  const char* vbase = reinterpret_cast<const char*>(ks) + (4 * hh + (i16 >> 2)) * pitchB +
+                      (D + 16 * (g16 & 1) + 4 * (i16 & 3)) * 2;
+  const float* bias = a.bias ? a.bias + myh : nullptr;
+  for (int j0 = jlo; j0 <= jhi; j0 += MKT) {
+    __syncthreads();  // every wave is done with the previous tile (first: the queries are being written)
+#pragma unroll
+    for (int u = 0; u < NPF; ++u) {
+      const int idx = tid + u * NT;
+      if (idx < nchunks) *reinterpret_cast<uint4*>(ks + (idx / kch) * KP + 8 * (idx % kch)) = pf[u];
+    }
+    __syncthreads();
+    if (j0 + MKT <= jhi) fetch(j0 + MKT, bt_lds);  // in flight while this tile is computed
+    if (!wave_live) continue;
+    f32x16_t sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    const bf16_t* ka = ks + qcol * KP + 8 * hh;
+    const bf16_t* qb = qs + (wave * 32 + qcol) * QP + 8 * hh;
+    for (int kk = 0; kk < nkk; ++kk) {
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(ka + 16 * kk));
+      const bf16x8_t bfr = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(qb + 16 * kk));
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr, sc, 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+      const int n = prow - j;
+      const bool valid = rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window);
+      float v = sc[r] * sl2;
+      if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+      v = valid ? v : -INFINITY;
+      sc[r] = v;
+      mx = fmaxf(mx, v);
+    }
+    mx = xor32_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float alpha = exp2f(m - mn);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float pe = exp2f(sc[r] - mn);
+      sc[r] = pe;
+      sum += pe;
+    }
+    sum = xor32_sum(sum);
+    l = l * alpha + sum;
+    m = mn;
+    bf16x8_t pfr[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      uint4 w;
+      w.x = pack2(sc[8 * s2 + 0], sc[8 * s2 + 1]);
+      w.y = pack2(sc[8 * s2 + 2], sc[8 * s2 + 3]);
+      w.z = pack2(sc[8 * s2 + 4], sc[8 * s2 + 5]);
+      w.w = pack2(sc[8 * s2 + 6], sc[8 * s2 + 7]);
+      pfr[s2] = __builtin_bit_cast(bf16x8_t, w);
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      if (alpha != 1.0f) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const char* a0 = vbase + (16 * s2) * pitchB + 64 * db;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(a0 + 8 * pitchB));
+        const short8_t a8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a8), pfr[s2], o[db], 0, 0, 0);
+      }
+    }
+  }
+  if (!rok) return;
+  if (nsplit > 1) {
+    float* wo = ws_o + ((int64_t)z * wrows + orow) * DV;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<float4*>(wo + 32 * db + 8 * q4 + 4 * hh) =
+            make_float4(o[db][4 * q4], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]);
+    if (hh == 0) {
+      ws_ml[((int64_t)z * wrows + orow) * 2] = m;
+      ws_ml[((int64_t)z * wrows + orow) * 2 + 1] = l;
+    }
+    return;
+  }
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  bf16_t* op = reinterpret_cast<bf16_t*>(a.out) + orow * DV;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      uint2 w;
+      w.x = pack2(o[db][4 * q4 + 0] * inv, o[db][4 * q4 + 1] * inv);
+      w.y = pack2(o[db][4 * q4 + 2] * inv, o[db][4 * q4 + 3] * inv);
+      *reinterpret_cast<uint2*>(op + 32 * db + 8 * q4 + 4 * hh) = w;
+    }
+  }
+}
+
+// out[row] = sum_z O_z 2^(m_z - m*) / sum_z l_z 2^(m_z - m*), m* = max_z m_z (running maxima in log2 units).
+__global__ void __launch_bounds__(128) sink_attn_merge_kernel(bf16_t* out, const float* ws_o, const float* ws_ml,
+                                                              int nsplit, int64_t rows, int DV) {
+  const int64_t row = blockIdx.x;
+  float mstar = -1e30f;
+  for (int z = 0; z < nsplit; ++z) mstar = fmaxf(mstar, ws_ml[((int64_t)z * rows + row) * 2]);
+  float lsum = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
+    if (lz > 0.f) lsum += lz * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
+  }
+  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  for (int c = threadIdx.x; c < DV; c += 128) {
+    float acc = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
+      if (lz > 0.f) acc += ws_o[((int64_t)z * rows + row) * DV + c] * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
+    }
+    out[row * DV + c] = f2bf(acc * inv);
+  }
+}
+
+template <int NDB, int NW, int NKC> hipError_t launch_mfma(const SinkAttnArgs& a, hipStream_t s) {
+  auto* fn = sink_attn_mfma_kernel<NDB, NW, NKC>;
+  const int kp = a.dim + a.vdim + 8, qp = a.dim + 8;
+  const size_t lds = sizeof(bf16_t) * ((size_t)32 * NW * qp + (size_t)MKT * kp) + sizeof(int) * BT_LDS_MAX;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       96 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const int qpg = a.heads / a.kv_heads;
+  const int nsplit = a.ws_o != nullptr ? max(1, a.nsplit) : 1;
+  const dim3 grid((unsigned)(((int64_t)a.max_q * qpg + 32 * NW - 1) / (32 * NW)), (unsigned)a.num_seqs,
+                  (unsigned)(a.kv_heads * nsplit));
+  hipLaunchKernelGGL(fn, grid, dim3(64 * NW), lds, s, a, kp, qp, a.ws_o, a.ws_ml, nsplit, a.chunk);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || nsplit <= 1) return e;
+  hipLaunchKernelGGL(sink_attn_merge_kernel, dim3((unsigned)((int64_t)a.heads * a.total_q)), dim3(128), 0, s,
+                     reinterpret_cast<bf16_t*>(a.out), a.ws_o, a.ws_ml, nsplit, (int64_t)a.heads * a.total_q, a.vdim);
+  return hipGetLastError();
+}
+
+template <int NW, int NKC> hipError_t launch_mfma_ndb(const SinkAttnArgs& a, hipStream_t s) {
+  switch (a.vdim / 32) {
+    case 1: return launch_mfma<1, NW, NKC>(a, s);
+    case 2: return launch_mfma<2, NW, NKC>(a, s);
+    case 3: return launch_mfma<3, NW, NKC>(a, s);
+    case 4: return launch_mfma<4, NW, NKC>(a, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <int NW> hipError_t launch_mfma_nw(const SinkAttnArgs& a, hipStream_t s) {
+  return a.dim <= 64 ? launch_mfma_ndb<NW, 8>(a, s) : launch_mfma_ndb<NW, 16>(a, s);
+}
+
+inline bool mfma_ok(const SinkAttnArgs& a) {
+  return !a.f32 && a.dim % 16 == 0 && a.dim <= 128 && a.vdim % 32 == 0 && a.vdim <= 128 &&
+         (reinterpret_cast<uintptr_t>(a.q) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.out) & 7) == 0;
+}
+
 }  // namespace
 
-bool sink_attn_uses_mfma(const SinkAttnArgs&) { return false; }
+bool sink_attn_uses_mfma(const SinkAttnArgs& a) { return a.impl != 1 && mfma_ok(a); }
 
 hipError_t launch_sink_attn(const SinkAttnArgs& a, hipStream_t s) {
   if (a.num_seqs == 0 || a.total_q == 0) return hipSuccess;
   if (a.heads < 1 || a.kv_heads < 1 || a.heads % a.kv_heads != 0 || a.dim < 1 || a.dim > 512 || a.vdim < 1 ||
       a.vdim > 256 || a.block_size < 1 || a.max_q < 1 || (a.bias != nullptr && a.bias_rows < 1))
     return hipErrorInvalidValue;
+  if (sink_attn_uses_mfma(a)) {
+    const int qpg = a.heads / a.kv_heads;
+    return a.max_q * qpg <= 32 ? launch_mfma_nw<1>(a, s) : launch_mfma_nw<4>(a, s);
+  }
   if (a.impl == 2) return hipErrorInvalidValue;
   return a.f32 ? launch_fma<true>(a, s) : launch_fma<false>(a, s);
 }

@@ -381,6 +381,8 @@ class LLMEngine:
             return None
         if getattr(self.model, "tp", None) is not None and self.model.tp.enabled:
             return None
+        if not any(getattr(c.seq, "export_kv", False) for c in chunks):
+            return None  # nothing exports (pools with rows of several widths have no planes to export from)
         planes = self.pool.planes()
         targets = []
         for c in chunks:

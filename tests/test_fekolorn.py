@@ -309,7 +309,7 @@ def _paged(device, dtype, n_blocks, bs, width, seed):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", ["rotary", "biased", "wide"])
+@pytest.mark.parametrize("case", ["rotary", "biased", "wide", "mc_rotary", "mc_biased"])
 def test_attention_ops_with_standout_keys(device, dtype, case):
     """qkv_prep + sink_attn over scattered pages, prompt portion and single decode rows: one key far back, one on a
     page border, and the keys just inside and just outside the window are made to stand out (their scores lead by
@@ -322,8 +322,14 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
         H, G, d, dv, window, rot, bias_max = 4, 2, 16, 8, 0, 8, 0
     elif case == "biased":
         H, G, d, dv, window, rot, bias_max = 6, 2, 12, 20, 21, 0, 15.0
+    elif case == "mc_rotary":     # shapes the matrix-core kernel takes in bf16 (forced there: impl 2)
+        H, G, d, dv, window, rot, bias_max = 8, 2, 80, 32, 0, 48, 0
+    elif case == "mc_biased":
+        H, G, d, dv, window, rot, bias_max = 6, 2, 32, 96, 37, 0, 15.0
     else:
         H, G, d, dv, window, rot, bias_max = 2, 1, 96, 160, 40, 0, 0
+    impl = 2 if case.startswith("mc_") and dtype == torch.bfloat16 and device != "cpu" else 0
+    rotary, biased = case.endswith("rotary"), case.endswith("biased")
     T, bs = 90, 8
     g = torch.Generator().manual_seed(len(case))
     q = torch.randn(T, H, d, generator=g) * 0.3
@@ -341,10 +347,10 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
     sink = torch.randn(H, generator=g)
     scale = d ** -0.5
     rel = torch.randn(10, H, generator=g) if bias_max else None
-    qn = (torch.rand(H * d, generator=g) + 0.5) if case == "biased" else None
-    kn = (torch.rand(G * d, generator=g) + 0.5) if case == "biased" else None
-    v_first = torch.randn(T, G * dv, generator=g) if case == "biased" else None
-    lam = torch.tensor([0.35]) if case == "biased" else None
+    qn = (torch.rand(H * d, generator=g) + 0.5) if biased else None
+    kn = (torch.rand(G * d, generator=g) + 0.5) if biased else None
+    v_first = torch.randn(T, G * dv, generator=g) if biased else None
+    lam = torch.tensor([0.35]) if biased else None
     qd, kd, vd = q.to(dtype).double(), k.to(dtype).double(), v.to(dtype).double()
     # oracle
     oq, ok_, ov = qd, kd, vd
@@ -354,7 +360,7 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
         ov = ((1 - 0.35) * vd.reshape(T, -1) + 0.35 * v_first.to(dtype).double()).view(T, G, dv)
     if rot:
         oq, ok_ = orc.rotate_half(oq, rot, 50.0), orc.rotate_half(ok_, rot, 50.0)
-    if case == "rotary":
+    if rotary:
         ov = orc.rms(ov, eps)
     bias = None
     if rel is not None:
@@ -379,12 +385,12 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
         slots = torch.tensor([perm[t // bs] * bs + t % bs for t in range(lo, hi)], device=device)
         p = proj[lo:hi]
         qr = seq.qkv_prep(p[:, :nq], p[:, nq: nq + nk], p[:, nq + nk:], cache, H, G, d, dv, pos, slots, eps,
-                          q_norm=dev(qn), k_norm=dev(kn), rot_dims=rot, inv_freq=inv_freq, v_unit=case == "rotary",
+                          q_norm=dev(qn), k_norm=dev(kn), rot_dims=rot, inv_freq=inv_freq, v_unit=rotary,
                           v_lambda=dev(lam), v_first=None if v_first is None else v_first[lo:hi].to(dtype).to(device))
         single = hi - lo == 1
         o = seq.sink_attn(qr, cache, bt, None if single else torch.tensor([0, hi - lo], dtype=torch.int32, device=device),
                           torch.tensor([hi], dtype=torch.int32, device=device), pos, sink.to(device), table,
-                          hi - lo, H, G, d, dv, window, scale)
+                          hi - lo, H, G, d, dv, window, scale, impl=impl)
         outs.append(o.cpu().double())
     got = torch.cat(outs)
     tol = 3e-4 if dtype == torch.float32 else 4e-2
