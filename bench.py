@@ -127,6 +127,10 @@ def parse(argv=None):
                    help="instead of the serving bench: Datatar beside the closest existing model (Mixtral) at equal "
                         "sizes, prefill / decode throughput and the attention kernels alone (bench/design_compare.py)")
     p.add_argument("--design-args", default="", help="arguments passed on to bench/design_compare.py")
+    p.add_argument("--fekolorn-compare", action="store_true",
+                   help="instead of the serving bench: Fekolorn beside the closest existing model (Llama) at equal "
+                        "sizes, prefill / decode throughput and its kernels alone (bench/fekolorn_compare.py)")
+    p.add_argument("--fekolorn-args", default="", help="arguments passed on to bench/fekolorn_compare.py")
     return p.parse_args(argv)
 
 
@@ -466,6 +470,15 @@ def main(argv=None) -> int:
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         return mod.main(shlex.split(args.design_args))
+    if args.fekolorn_compare:  # likewise a separate measurement
+        import importlib.util
+        import shlex
+
+        spec = importlib.util.spec_from_file_location("fekolorn_compare",
+                                                      os.path.join(ROOT, "bench", "fekolorn_compare.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod.main(shlex.split(args.fekolorn_args))
     if needs_launcher(args):
         return self_launch(args, argv)
     world = int(os.environ.get("WORLD_SIZE", "1"))

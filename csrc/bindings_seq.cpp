@@ -335,7 +335,7 @@ void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTenso
   a.chunk = 0;
   Tensor ws_o, ws_ml;
   if (die::sink_attn_uses_mfma(a)) {
-    // few row tiles (decode steps): split the keys over workgroups until about 512 are in flight. The key range is
+    // few row tiles (decode steps): split the keys over workgroups until about 2048 are in flight. The key range is
     // bounded by the window, else by the block table's width (under a captured graph: the model length; splits
     // beyond a sequence's keys exit at once)
     const int64_t qpg = heads / kv_heads;
@@ -343,7 +343,7 @@ void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTenso
     const int64_t tiles = S * kv_heads * ((max_q * qpg + rows_wg - 1) / rows_wg);
     int64_t bound = block_tables.size(1) * cache.size(1);
     if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
-    const int64_t ns = std::min<int64_t>({(int64_t)16, 512 / std::max<int64_t>(1, tiles), (bound + 127) / 128});
+    const int64_t ns = std::min<int64_t>({(int64_t)16, 2048 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
     if (ns > 1) {
       a.chunk = (int)((((bound + ns - 1) / ns) + 31) / 32 * 32);
       a.nsplit = (int)((bound + a.chunk - 1) / a.chunk);

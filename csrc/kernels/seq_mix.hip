@@ -8,7 +8,8 @@
 //   poly_norm_act       c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3
 //   delta_prep          short conv + SiLU of q/k/v, unit q/k, beta and decay of the gated delta rule
 //   conv_state_update   the convolution's trailing inputs -> state
-//   gated_delta         the recurrence itself, one workgroup per (sequence, head), state columns in registers
+//   gated_delta         the recurrence itself, one workgroup per (sequence, head), the state in registers (a
+//                       column per lane quad)
 //   qkv_prep            q/k norm, rotate-half rotary, value norm / value mixing, paged cache write
 #include "common.h"
 #include "seq_launchers.h"
@@ -31,6 +32,26 @@ __device__ __forceinline__ float rnd(float v, bool f32) { return f32 ? v : bf2f(
 __device__ __forceinline__ float siluf(float z) { return z / (1.0f + expf(-z)); }
 
 constexpr int NT = 256;
+
+__device__ __forceinline__ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+__device__ __forceinline__ bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; }
+// 4 consecutive values (element index i a multiple of 4, the address 8- or 16-byte aligned)
+__device__ __forceinline__ float4 ld4(const void* p, int64_t i, bool f32) {
+  if (f32) return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const bf16_t*>(p) + i);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                     __uint_as_float(w.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4(void* p, int64_t i, bool f32, float4 v, float sc) {
+  if (f32) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p) + i) = make_float4(v.x * sc, v.y * sc, v.z * sc, v.w * sc);
+  } else {
+    uint2 w;
+    w.x = pack2(v.x * sc, v.y * sc);
+    w.y = pack2(v.z * sc, v.w * sc);
+    *reinterpret_cast<uint2*>(reinterpret_cast<bf16_t*>(p) + i) = w;
+  }
+}
 
 // sequence of a row: the largest s with cu_q[s] <= row (cu_q == nullptr: the row itself)
 __device__ __forceinline__ int seq_of_row(const int* cu_q, int num_seqs, int row) {
@@ -98,6 +119,83 @@ __global__ void __launch_bounds__(NT) stream_mix_norm_kernel(StreamMixArgs a) {
   const int64_t t = blockIdx.x;
   float* xs = a.streams + t * S * W;
   float ss = 0.f;
+  // rows of a multiple of 4 columns: 16-byte accesses, 4 columns per thread and trip; the first KEEP trips keep
+  // their u = in . x in registers for the second pass (widths up to 4 * KEEP * NT), later ones re-read the streams
+  const bool y_ok = a.y1 == nullptr || (a.ys1 % 4 == 0 && aligned8(a.y1) && (a.y2 == nullptr || (a.ys2 % 4 == 0 && aligned8(a.y2))));
+  if (W % 4 == 0 && aligned16(a.streams) && y_ok && (a.h == nullptr || aligned16(a.h))) {
+    constexpr int KEEP = 8;
+    const int W4 = W / 4;
+    float4 ukeep[KEEP];
+    auto trip = [&](int c4) -> float4 {
+      float4 x[SMAX];
+#pragma unroll
+      for (int s = 0; s < SMAX; ++s)
+        if (s < S) x[s] = reinterpret_cast<const float4*>(xs + (int64_t)s * W)[c4];
+      float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (a.y1 != nullptr) {
+        float4 y = ld4(a.y1, t * a.ys1 + 4 * c4, a.y_f32);
+        y.x *= a.a1, y.y *= a.a1, y.z *= a.a1, y.w *= a.a1;
+        if (a.y2 != nullptr) {
+          const float4 y2 = ld4(a.y2, t * a.ys2 + 4 * c4, a.y_f32);
+          y.x += a.a2 * y2.x, y.y += a.a2 * y2.y, y.z += a.a2 * y2.z, y.w += a.a2 * y2.w;
+        }
+#pragma unroll
+        for (int to = 0; to < SMAX; ++to) {
+          if (to < S) {
+            const float ow = outw[to];
+            float4 n = make_float4(ow * y.x, ow * y.y, ow * y.z, ow * y.w);
+#pragma unroll
+            for (int s = 0; s < SMAX; ++s) {
+              if (s < S) {
+                const float m = mixw[s * S + to];
+                n.x += m * x[s].x, n.y += m * x[s].y, n.z += m * x[s].z, n.w += m * x[s].w;
+              }
+            }
+            reinterpret_cast<float4*>(xs + (int64_t)to * W)[c4] = n;
+            const float iw = inw[to];
+            u.x += iw * n.x, u.y += iw * n.y, u.z += iw * n.z, u.w += iw * n.w;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+          if (s < S) {
+            const float iw = inw[s];
+            u.x += iw * x[s].x, u.y += iw * x[s].y, u.z += iw * x[s].z, u.w += iw * x[s].w;
+          }
+        }
+      }
+      ss += u.x * u.x + u.y * u.y + u.z * u.z + u.w * u.w;
+      return u;
+    };
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+      const int c4 = it * NT + threadIdx.x;
+      if (c4 < W4) ukeep[it] = trip(c4);
+    }
+    for (int c4 = KEEP * NT + threadIdx.x; c4 < W4; c4 += NT) trip(c4);
+    if (a.h == nullptr) return;
+    ss = block_sum<NT>(ss, red);
+    const float rs = a.gain[0] / sqrtf(ss / (float)W + a.eps);
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+      const int c4 = it * NT + threadIdx.x;
+      if (c4 < W4) st4(a.h, t * W + 4 * c4, a.h_f32, ukeep[it], rs);
+    }
+    for (int c4 = KEEP * NT + threadIdx.x; c4 < W4; c4 += NT) {
+      float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int s = 0; s < SMAX; ++s) {
+        if (s < S) {
+          const float4 x = reinterpret_cast<const float4*>(xs + (int64_t)s * W)[c4];  // this thread's own writes
+          const float iw = inw[s];
+          u.x += iw * x.x, u.y += iw * x.y, u.z += iw * x.z, u.w += iw * x.w;
+        }
+      }
+      st4(a.h, t * W + 4 * c4, a.h_f32, u, rs);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < W; c += NT) {
     float x[SMAX];
 #pragma unroll
@@ -141,6 +239,46 @@ __global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void
   __shared__ float red[NT / 64];
   const int64_t r = blockIdx.x;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  // bf16 rows of a multiple of 8 columns, up to 8 * KEEP * NT wide: 16-byte accesses, the row kept in registers
+  constexpr int KEEP = 4;
+  if (!f32 && n % 8 == 0 && n <= 8 * KEEP * NT && zstride % 8 == 0 && aligned16(z) && aligned16(out)) {
+    const uint4* zr = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(z) + r * zstride);
+    uint4 keep[KEEP];
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+      const int c8 = it * NT + threadIdx.x;
+      if (c8 < n / 8) {
+        keep[it] = zr[c8];
+        float f[8];
+        unpack8(keep[it], f);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const float v2 = f[q] * f[q];
+          s2 += v2;
+          s4 += v2 * v2;
+          s6 += v2 * v2 * v2;
+        }
+      }
+    }
+    s2 = block_sum<NT>(s2, red);
+    s4 = block_sum<NT>(s4, red);
+    s6 = block_sum<NT>(s6, red);
+    const float r1 = coef[0] / sqrtf(s2 / (float)n + eps), r2 = coef[1] / sqrtf(s4 / (float)n + eps),
+                r3 = coef[2] / sqrtf(s6 / (float)n + eps), c3 = coef[3];
+    uint4* orow = reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(out) + r * n);
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+      const int c8 = it * NT + threadIdx.x;
+      if (c8 < n / 8) {
+        float f[8];
+        unpack8(keep[it], f);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] = f[q] * r1 + f[q] * f[q] * r2 + f[q] * f[q] * f[q] * r3 + c3;
+        orow[c8] = pack8(f);
+      }
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < n; c += NT) {
     const float v = ldv(z, r * zstride + c, f32);
     const float v2 = v * v;
@@ -240,72 +378,97 @@ __global__ void __launch_bounds__(NT) conv_state_update_kernel(float* conv_state
 
 constexpr int TB = 16;  // tokens staged per trip
 
-template <int DM>
-__global__ void __launch_bounds__(256) gated_delta_kernel(void* out, const float* qkv32, const float* bg,
-                                                         const void* gate, int64_t gstride, bool f32,
-                                                         const float* norm_w, float eps, float* state, DeltaShape sh,
-                                                         RaggedRows r) {
-  extern __shared__ float sm[];
+// One workgroup per (sequence, head). The state S [dim, vdim] lives in registers for the whole step: column j is
+// split over the 4 lanes of a quad, lane `part` holding rows [part * DP, (part + 1) * DP) — so a token costs each
+// lane 3 * DP multiply-adds and two quad reductions (S^T k and S^T q), with q and k read from LDS as float4
+// broadcasts, and 4 * vdim lanes work on one head. Tokens are staged TB at a time; the read-outs of a trip are
+// normed and gated afterwards, one wave per token.
+template <int DP>
+__global__ void __launch_bounds__(1024) gated_delta_kernel(void* out, const float* qkv32, const float* bg,
+                                                          const void* gate, int64_t gstride, bool f32,
+                                                          const float* norm_w, float eps, float* state, DeltaShape sh,
+                                                          RaggedRows r) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  constexpr int DPAD = 4 * DP;
   const int d = sh.dim, dv = sh.vdim, H = sh.heads, G = sh.kv_heads, C = sh.channels();
-  float* qs = sm;               // [TB][d]
-  float* ks = qs + TB * d;      // [TB][d]
-  float* vs = ks + TB * d;      // [TB][dv]
-  float* os = vs + TB * dv;     // [TB][dv]
-  float* bs = os + TB * dv;     // [TB] beta
-  float* gs = bs + TB;          // [TB] decay
-  const int h = blockIdx.x, s = blockIdx.y, j = threadIdx.x, nthr = blockDim.x;
+  float* qs = sm;                  // [TB][DPAD], zero beyond dim
+  float* ks = qs + TB * DPAD;      // [TB][DPAD]
+  float* vs = ks + TB * DPAD;      // [TB][dv]
+  float* os = vs + TB * dv;        // [TB][dv]
+  float* bs = os + TB * dv;        // [TB] beta
+  float* gs = bs + TB;             // [TB] decay
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
+  const int j = tid >> 2, part = tid & 3;
   const int kh = h / (H / G);
   const int q0 = r.cu_q ? r.cu_q[s] : s;
   const int L = r.cu_q ? r.cu_q[s + 1] - q0 : 1;
   if (L <= 0) return;
   const bool fresh = r.positions[q0] <= 0;
   float* st = state + ((int64_t)r.state_slots[s] * H + h) * d * dv;
-  float S[DM];
+  float S[DP];
 #pragma unroll
-  for (int i = 0; i < DM; ++i) S[i] = (!fresh && i < d && j < dv) ? st[(int64_t)i * dv + j] : 0.f;
-  const int lane = j & 63, wave = j >> 6, nwaves = nthr >> 6;
+  for (int i = 0; i < DP; ++i) {
+    const int row = part * DP + i;
+    S[i] = (!fresh && row < d && j < dv) ? st[(int64_t)row * dv + j] : 0.f;
+  }
+  const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
   for (int t0 = 0; t0 < L; t0 += TB) {
     const int nb = min(TB, L - t0);
     __syncthreads();
-    for (int e = j; e < nb * d; e += nthr) {
-      const int tt = e / d, c = e % d;
+    for (int e = tid; e < nb * DPAD; e += nthr) {
+      const int tt = e / DPAD, c = e % DPAD;
       const float* row = qkv32 + (int64_t)(q0 + t0 + tt) * C;
-      qs[tt * d + c] = row[kh * d + c];
-      ks[tt * d + c] = row[G * d + kh * d + c];
+      qs[e] = c < d ? row[kh * d + c] : 0.f;
+      ks[e] = c < d ? row[G * d + kh * d + c] : 0.f;
     }
-    for (int e = j; e < nb * dv; e += nthr) {
+    for (int e = tid; e < nb * dv; e += nthr) {
       const int tt = e / dv, c = e % dv;
-      vs[tt * dv + c] = qkv32[(int64_t)(q0 + t0 + tt) * C + 2 * G * d + h * dv + c];
+      vs[e] = qkv32[(int64_t)(q0 + t0 + tt) * C + 2 * G * d + h * dv + c];
     }
-    if (j < nb) {
-      bs[j] = bg[(int64_t)(q0 + t0 + j) * 2 * H + h];
-      gs[j] = bg[(int64_t)(q0 + t0 + j) * 2 * H + H + h];
+    if (tid < nb) {
+      bs[tid] = bg[(int64_t)(q0 + t0 + tid) * 2 * H + h];
+      gs[tid] = bg[(int64_t)(q0 + t0 + tid) * 2 * H + H + h];
     }
     __syncthreads();
-    if (j < dv) {
-      for (int tt = 0; tt < nb; ++tt) {
-        const float g = gs[tt], beta = bs[tt];
-        const float* kt = ks + tt * d;
-        const float* qt = qs + tt * d;
-        float dot = 0.f;
+    for (int tt = 0; tt < nb; ++tt) {
+      const float g = gs[tt], beta = bs[tt];
+      const float4* kt = reinterpret_cast<const float4*>(ks + tt * DPAD + part * DP);
+      const float4* qt = reinterpret_cast<const float4*>(qs + tt * DPAD + part * DP);
+      float kreg[DP];
+      float d0 = 0.f, d1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < DM; ++i) {
-          if (i < d) {
-            S[i] *= g;
-            dot += S[i] * kt[i];
-          }
-        }
-        const float u = beta * (vs[tt * dv + j] - dot);
-        float o = 0.f;
-#pragma unroll
-        for (int i = 0; i < DM; ++i) {
-          if (i < d) {
-            S[i] += kt[i] * u;
-            o += S[i] * qt[i];
-          }
-        }
-        os[tt * dv + j] = o;
+      for (int i = 0; i < DP / 4; ++i) {
+        const float4 k4 = kt[i];
+        kreg[4 * i] = k4.x;
+        kreg[4 * i + 1] = k4.y;
+        kreg[4 * i + 2] = k4.z;
+        kreg[4 * i + 3] = k4.w;
+        S[4 * i] *= g;
+        S[4 * i + 1] *= g;
+        S[4 * i + 2] *= g;
+        S[4 * i + 3] *= g;
+        d0 += S[4 * i] * k4.x + S[4 * i + 2] * k4.z;
+        d1 += S[4 * i + 1] * k4.y + S[4 * i + 3] * k4.w;
       }
+      float dot = d0 + d1;
+      dot += __shfl_xor(dot, 1, 64);
+      dot += __shfl_xor(dot, 2, 64);
+      const float u = beta * ((j < dv ? vs[tt * dv + j] : 0.f) - dot);
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DP / 4; ++i) {
+        const float4 q4 = qt[i];
+        S[4 * i] += kreg[4 * i] * u;
+        S[4 * i + 1] += kreg[4 * i + 1] * u;
+        S[4 * i + 2] += kreg[4 * i + 2] * u;
+        S[4 * i + 3] += kreg[4 * i + 3] * u;
+        o0 += S[4 * i] * q4.x + S[4 * i + 2] * q4.z;
+        o1 += S[4 * i + 1] * q4.y + S[4 * i + 3] * q4.w;
+      }
+      float o = o0 + o1;
+      o += __shfl_xor(o, 1, 64);
+      o += __shfl_xor(o, 2, 64);
+      if (part == 0 && j < dv) os[tt * dv + j] = o;
     }
     __syncthreads();
     for (int tt = wave; tt < nb; tt += nwaves) {
@@ -322,8 +485,10 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(void* out, const float
   }
   if (j < dv) {
 #pragma unroll
-    for (int i = 0; i < DM; ++i)
-      if (i < d) st[(int64_t)i * dv + j] = S[i];
+    for (int i = 0; i < DP; ++i) {
+      const int row = part * DP + i;
+      if (row < d) st[(int64_t)row * dv + j] = S[i];
+    }
   }
 }
 
@@ -463,17 +628,17 @@ hipError_t launch_conv_state_update(float* conv_state, const void* x, int64_t xs
   return hipGetLastError();
 }
 
-template <int DM>
+template <int DP>
 static hipError_t launch_gd(void* out, const float* qkv32, const float* bg, const void* gate, int64_t gstride, bool f32,
                             const float* norm_w, float eps, float* state, DeltaShape sh, RaggedRows r, hipStream_t s) {
-  const int nthr = (sh.vdim + 63) / 64 * 64;
-  const size_t lds = sizeof(float) * (TB * (2 * sh.dim + 2 * sh.vdim) + 2 * TB);
+  const int nthr = (4 * sh.vdim + 63) / 64 * 64;
+  const size_t lds = sizeof(float) * (TB * (2 * 4 * DP + 2 * sh.vdim) + 2 * TB);
   if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gated_delta_kernel<DM>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gated_delta_kernel<DP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(gated_delta_kernel<DM>, dim3(sh.heads, r.num_seqs), dim3(nthr), lds, s, out, qkv32, bg, gate,
+  hipLaunchKernelGGL(gated_delta_kernel<DP>, dim3(sh.heads, r.num_seqs), dim3(nthr), lds, s, out, qkv32, bg, gate,
                      gstride, f32, norm_w, eps, state, sh, r);
   return hipGetLastError();
 }
@@ -483,10 +648,12 @@ hipError_t launch_gated_delta(void* out, const float* qkv32, const float* bg, co
                               hipStream_t s) {
   if (r.num_seqs == 0 || r.total_rows == 0) return hipSuccess;
   if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
-  if (sh.dim <= 32) return launch_gd<32>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
-  if (sh.dim <= 64) return launch_gd<64>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
-  if (sh.dim <= 128) return launch_gd<128>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
-  return launch_gd<256>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  // rows of the state per lane of a quad: dim / 4, rounded up to a multiple of 4
+  if (sh.dim <= 16) return launch_gd<4>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  if (sh.dim <= 32) return launch_gd<8>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  if (sh.dim <= 64) return launch_gd<16>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  if (sh.dim <= 128) return launch_gd<32>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
+  return launch_gd<64>(out, qkv32, bg, gate, gstride, f32, norm_w, eps, state, sh, r, s);
 }
 
 hipError_t launch_qkv_prep(const QkvPrepArgs& a, hipStream_t s) {

@@ -203,13 +203,15 @@ def test_embedding_with_previous_token_state(device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("S", [1, 3, 8])
-def test_stream_mixing_and_norm(device, dtype, S):
+@pytest.mark.parametrize("S,W", [(1, 37), (3, 37), (8, 37), (3, 64), (2, 8448)])
+def test_stream_mixing_and_norm(device, dtype, S, W):
+    """Narrow rows (scalar accesses), rows of a multiple of 4 columns (16-byte accesses), and rows wider than what
+    the kernel keeps in registers between its two passes."""
     _need(device)
     from src.ops import seq
 
     g = torch.Generator().manual_seed(S)
-    T, W, eps = 5, 37, 1e-4
+    T, eps = 5, 1e-4
     xs = torch.randn(T, S, W, generator=g)
     y1, y2 = torch.randn(T, W, generator=g).to(dtype), torch.randn(T, W, generator=g).to(dtype)
     mixw, outw, inw = torch.randn(S, S, generator=g), torch.randn(S, generator=g), torch.randn(S, generator=g)
@@ -245,8 +247,23 @@ def test_polynomial_norm_activation(device, n):
     want = 0.7 * orc.rms(zz, 1e-5) - 0.3 * orc.rms(zz ** 2, 1e-5) + 0.2 * orc.rms(zz ** 3, 1e-5) + 0.05
     got = seq.poly_norm_act(z.to(device), coef.to(device), 1e-5)
     assert torch.allclose(got.cpu().double(), want, atol=1e-4)
-    big = torch.cat([z, z.new_zeros(4, 8)], 1)[:, :n].to(device)   # a strided view is not needed: rows are dense
-    assert torch.allclose(seq.poly_norm_act(big, coef.to(device), 1e-5).cpu().double(), want, atol=1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("n", [64, 4096, 8200])
+def test_polynomial_norm_activation_bf16_rows(device, n):
+    """bf16 rows: 16-byte accesses with the row kept in registers, and rows too wide for that."""
+    _need(device)
+    from src.ops import seq
+
+    g = torch.Generator().manual_seed(n)
+    z = (torch.randn(3, n, generator=g) * 1.5).bfloat16()
+    coef = torch.tensor([0.7, -0.3, 0.2, 0.05])
+    zz = z.double()
+    want = 0.7 * orc.rms(zz, 1e-5) - 0.3 * orc.rms(zz ** 2, 1e-5) + 0.2 * orc.rms(zz ** 3, 1e-5) + 0.05
+    got = seq.poly_norm_act(z.to(device), coef.to(device), 1e-5)
+    assert got.dtype == torch.bfloat16
+    assert float((got.cpu().double() - want).abs().max()) < 2e-2 * max(1.0, float(want.abs().max()))
 
 
 def _delta_weights(H, G, d, dv, taps, W, seed):
