@@ -274,6 +274,7 @@ void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, Tensor v, int64_t 
   a.slots = slots.data_ptr<int64_t>();
   a.q_out = q_out.data_ptr();
   a.cache = cache.data_ptr();
+  a.block_size = (int)cache.size(1);
   HIP_OK(die::launch_qkv_prep(a, cur_stream()));
 }
 

@@ -96,14 +96,15 @@ struct QkvPrepArgs {
   const int64_t* positions;
   const int64_t* slots;   // cache slot per row, < 0: not written
   void* q_out;            // [T, H * dim]
-  void* cache;            // [slots, G * dim + G * vdim] rows
+  void* cache;            // blocks of block_size tokens, head-major: [G][block_size][K: dim | V: vdim]
+  int block_size;
 };
 hipError_t launch_qkv_prep(const QkvPrepArgs& a, hipStream_t s);
 
 struct SinkAttnArgs {
   void* out;              // [T, H * vdim]
   const void* q;          // [T, H * dim]
-  const void* cache;      // [num_blocks, block_size, G * dim + G * vdim]
+  const void* cache;      // [num_blocks][G][block_size][K: dim | V: vdim]
   const int* block_tables;
   int bt_stride;
   const int* cu_q;        // nullptr: one row per sequence

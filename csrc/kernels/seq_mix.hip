@@ -556,8 +556,13 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
   for (int c = threadIdx.x; c < nq; c += NT) stv(a.q_out, t * nq + c, f32, qv[c]);
   const int64_t slot = a.slots[t];
   if (slot < 0) return;
-  const int64_t dst = slot * (int64_t)(nk + nv);
-  for (int c = threadIdx.x; c < nk + nv; c += NT) stv(a.cache, dst + c, f32, kv[c]);  // kv and vv are adjacent
+  // the block's interior is head-major: [G][block_size][K | V]
+  const int64_t blk = slot / a.block_size, off = slot % a.block_size;
+  for (int c = threadIdx.x; c < nk + nv; c += NT) {
+    const int g = c < nk ? c / d : (c - nk) / dv;
+    const int e = c < nk ? c % d : d + (c - nk) % dv;
+    stv(a.cache, ((blk * G + g) * a.block_size + off) * (int64_t)(d + dv) + e, f32, kv[c]);  // kv and vv are adjacent
+  }
 }
 
 bool rows_ok(const RaggedRows& r) { return r.positions != nullptr && r.state_slots != nullptr && r.num_seqs >= 0; }
@@ -659,7 +664,7 @@ hipError_t launch_gated_delta(void* out, const float* qkv32, const float* bg, co
 hipError_t launch_qkv_prep(const QkvPrepArgs& a, hipStream_t s) {
   if (a.T == 0) return hipSuccess;
   if (a.heads < 1 || a.kv_heads < 1 || a.heads % a.kv_heads != 0 || a.dim < 1 || a.vdim < 1 || a.rot_dims < 0 ||
-      a.rot_dims > a.dim || (a.rot_dims & 1) || (a.rot_dims > 0 && a.inv_freq == nullptr) ||
+      a.rot_dims > a.dim || (a.rot_dims & 1) || a.block_size < 1 || (a.rot_dims > 0 && a.inv_freq == nullptr) ||
       ((a.q_norm == nullptr) != (a.k_norm == nullptr)) || (a.v_lambda != nullptr && a.v_first == nullptr))
     return hipErrorInvalidValue;
   const size_t lds = sizeof(float) * ((size_t)a.heads * a.dim + (size_t)a.kv_heads * (a.dim + a.vdim));

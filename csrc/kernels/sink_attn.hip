@@ -1,5 +1,6 @@
-// Grouped-query softmax attention over a paged cache whose row per token is [K: G x dim | V: G x vdim], for prompt
-// portions and single decode tokens alike. A query at position p of its sequence sees the cached positions j <= p
+// Grouped-query softmax attention over a paged cache, for prompt portions and single decode tokens alike. A cache
+// block holds block_size tokens head-major: [G][block_size][K: dim | V: vdim], so the keys and values that one
+// key/value head reads from a block are one contiguous piece of memory. A query at position p of its sequence sees the cached positions j <= p
 // with p - j < window (window 0: all of them); its score is (q . k_j) * scale + bias[min(p - j, bias_rows - 1), h]
 // (bias optional); the softmax denominator holds one more per-head term exp(sink_h) that belongs to no position
 // (the running maximum starts at the sink, the running sum at 1). Query and value widths may differ.
@@ -42,7 +43,7 @@ __global__ void __launch_bounds__(256) sink_attn_kernel(SinkAttnArgs a, int QS, 
   float* ps = vs + BK * VS;         // [RW][BK]
   const int s = blockIdx.y, g = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int H = a.heads, G = a.kv_heads, QPG = H / G, D = a.dim, DV = a.vdim;
-  const int roww = G * (D + DV);
+  const int roww = D + DV;
   const int q0 = a.cu_q ? a.cu_q[s] : s;
   const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
   const int nrows = nq * QPG, row0 = blockIdx.x * RW;
@@ -87,9 +88,10 @@ __global__ void __launch_bounds__(256) sink_attn_kernel(SinkAttnArgs a, int QS, 
     for (int k = wave; k < BK; k += WAVES) {
       const int j = j0 + k;
       const bool in = j <= jhi;
-      const int64_t rowp = in ? ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * roww : 0;
-      for (int d = lane; d < D; d += 64) ks[k * KS + d] = in ? ldt<F32>(a.cache, rowp + g * D + d) : 0.f;
-      for (int d = lane; d < DV; d += 64) vs[k * VS + d] = in ? ldt<F32>(a.cache, rowp + G * D + g * DV + d) : 0.f;
+      const int64_t rowp =
+          in ? (((int64_t)bt[j / a.block_size] * G + g) * a.block_size + j % a.block_size) * roww : 0;
+      for (int d = lane; d < D; d += 64) ks[k * KS + d] = in ? ldt<F32>(a.cache, rowp + d) : 0.f;
+      for (int d = lane; d < DV; d += 64) vs[k * VS + d] = in ? ldt<F32>(a.cache, rowp + D + d) : 0.f;
     }
     __syncthreads();
     float acc[RPW];
@@ -205,13 +207,16 @@ typedef __attribute__((address_space(3))) short4_t lds_short4;
 typedef __attribute__((ext_vector_type(8))) short short8_t;
 
 template <int NDB, int NW, int NKC>
-__global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a, int KP, int QP, float* ws_o,
-                                                                float* ws_ml, int nsplit, int chunk) {
+__global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a, int KP, int QP, int QR, int BTC,
+                                                                float* ws_o, float* ws_ml, int nsplit, int chunk) {
   constexpr int ROWS = 32 * NW, NT = 64 * NW;
   constexpr int NPF = (MKT * (4 * NDB + NKC) + NT - 1) / NT;  // 16-byte chunks of a key tile per thread
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [ROWS][QP]
-  bf16_t* ks = qs + ROWS * QP;                                // [MKT][KP] = [K_g | V_g]
+  // QR query rows are staged: all ROWS of a prompt-sized step; for steps of few rows (NW = 1) only the rows there
+  // can be plus one zero row that every further query column reads, which keeps the workgroup's LDS small enough
+  // for two waves per SIMD
+  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);          // [QR][QP]
+  bf16_t* ks = qs + QR * QP;                                  // [MKT][KP] = [K_g | V_g]
   int bx = blockIdx.x, by = blockIdx.y;
   {
     // XCD k (workgroups are dealt round-robin by linear id) takes a contiguous eighth of the sequence-major tile
@@ -226,7 +231,7 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   const int H = a.heads, G = a.kv_heads, QPG = H / G, D = a.dim, DV = a.vdim;
   const int s = by, g = blockIdx.z % G, z = blockIdx.z / G;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
-  const int roww = G * (D + DV);
+  const int roww = D + DV;
   const int q0 = a.cu_q ? a.cu_q[s] : s;
   const int nq = a.cu_q ? a.cu_q[s + 1] - q0 : 1;
   const int nrows = nq * QPG, row0 = bx * ROWS;
@@ -257,7 +262,7 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   }
 
   const int lch = D / 8;
-  for (int idx = tid; idx < ROWS * lch; idx += NT) {
+  for (int idx = tid; idx < QR * lch; idx += NT) {
     const int r = idx / lch, c = idx % lch, row = row0 + r;
     uint4 v = make_uint4(0, 0, 0, 0);
     if (row < nrows) {
@@ -281,25 +286,34 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
 
   const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
-  const int kchK = D / 8, kch = (D + DV) / 8, nkk = D / 16, nchunks = MKT * kch;
+  const int kch = (D + DV) / 8, nkk = D / 16;
   int* btl = reinterpret_cast<int*>(ks + MKT * KP);
   const int b_lo = jlo / a.block_size, nbt = jhi / a.block_size - b_lo + 1;
-  const bool bt_lds = nbt <= BT_LDS_MAX;
+  const bool bt_lds = nbt <= BTC;
   if (bt_lds)
     for (int u = tid; u < nbt; u += NT) btl[u] = bt[b_lo + u];
   uint4 pf[NPF];
+  // chunk idx = tid + u * NT of a tile is (key k, 16-byte piece c) = (idx / kch, idx % kch): one division per
+  // thread, then steps of (NT / kch, NT % kch); a block size that is a power of two divides by shifting
+  const int k_first = tid / kch, c_first = tid - k_first * kch, k_step = NT / kch, c_step = NT - k_step * kch;
+  const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
   auto fetch = [&](int j0, bool lds) {
+    int k = k_first, c = c_first;
 #pragma unroll
     for (int u = 0; u < NPF; ++u) {
-      const int idx = tid + u * NT;
-      const int k = idx / kch, c = idx % kch, j = j0 + k;
+      const int j = j0 + k;
       pf[u] = make_uint4(0, 0, 0, 0);
-      if (idx < nchunks && j <= jhi) {
-        const int jb = j / a.block_size;
+      if (k < MKT && j <= jhi) {
+        const int jb = bs_shift >= 0 ? j >> bs_shift : j / a.block_size;
         const int64_t blk = lds ? btl[jb - b_lo] : bt[jb];
-        const int64_t rowp = (blk * a.block_size + (j - jb * a.block_size)) * roww;
-        const int64_t col = c < kchK ? (int64_t)g * D + 8 * c : (int64_t)G * D + (int64_t)g * DV + 8 * (c - kchK);
-        pf[u] = *reinterpret_cast<const uint4*>(cache + rowp + col);
+        const int64_t rowp = ((blk * G + g) * a.block_size + (j - jb * a.block_size)) * roww;
+        pf[u] = *reinterpret_cast<const uint4*>(cache + rowp + 8 * c);
+      }
+      k += k_step;
+      c += c_step;
+      if (c >= kch) {
+        c -= kch;
+        ++k;
       }
     }
   };
@@ -309,12 +323,25 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   const char* vbase = reinterpret_cast<const char*>(ks) + (4 * hh + (i16 >> 2)) * pitchB +
                       (D + 16 * (g16 & 1) + 4 * (i16 & 3)) * 2;
   const float* bias = a.bias ? a.bias + myh : nullptr;
+  // a tile is interior for a wave when every one of its 32 x 32 (key, row) pairs is visible: no masking then
+  const int wrow_first = row0 + wave * 32, wrow_last = wrow_first + 31;
+  const bool wave_full = wrow_last < nrows;
+  const int pw_first = wave_full ? (int)a.positions[q0 + wrow_first / QPG] : 0;
+  const int pw_last = wave_full ? (int)a.positions[q0 + wrow_last / QPG] : 0;
   for (int j0 = jlo; j0 <= jhi; j0 += MKT) {
     __syncthreads();  // every wave is done with the previous tile (first: the queries are being written)
+    {
+      int k = k_first, c = c_first;
 #pragma unroll
-    for (int u = 0; u < NPF; ++u) {
-      const int idx = tid + u * NT;
-      if (idx < nchunks) *reinterpret_cast<uint4*>(ks + (idx / kch) * KP + 8 * (idx % kch)) = pf[u];
+      for (int u = 0; u < NPF; ++u) {
+        if (k < MKT) *reinterpret_cast<uint4*>(ks + k * KP + 8 * c) = pf[u];
+        k += k_step;
+        c += c_step;
+        if (c >= kch) {
+          c -= kch;
+          ++k;
+        }
+      }
     }
     __syncthreads();
     if (j0 + MKT <= jhi) fetch(j0 + MKT, bt_lds);  // in flight while this tile is computed
@@ -323,31 +350,46 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
     const bf16_t* ka = ks + qcol * KP + 8 * hh;
-    const bf16_t* qb = qs + (wave * 32 + qcol) * QP + 8 * hh;
+    const bf16_t* qb = qs + min(wave * 32 + qcol, QR - 1) * QP + 8 * hh;
     for (int kk = 0; kk < nkk; ++kk) {
       const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(ka + 16 * kk));
       const bf16x8_t bfr = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(qb + 16 * kk));
       sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr, sc, 0, 0, 0);
     }
     float mx = -INFINITY;
+    const bool interior = wave_full && j0 + MKT - 1 <= min(pw_first, jhi) &&
+                          (a.window <= 0 || pw_last - j0 < a.window);
+    if (interior) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
-      const int n = prow - j;
-      const bool valid = rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window);
-      float v = sc[r] * sl2;
-      if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
-      v = valid ? v : -INFINITY;
-      sc[r] = v;
-      mx = fmaxf(mx, v);
+      for (int r = 0; r < 16; ++r) {
+        float v = sc[r] * sl2;
+        if (bias != nullptr) {
+          const int n = prow - (j0 + (r & 3) + 8 * (r >> 2) + 4 * hh);
+          v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+        }
+        sc[r] = v;
+        mx = fmaxf(mx, v);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+        const int n = prow - j;
+        const bool valid = rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window);
+        float v = sc[r] * sl2;
+        if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+        v = valid ? v : -INFINITY;
+        sc[r] = v;
+        mx = fmaxf(mx, v);
+      }
     }
     mx = xor32_max(mx);
     const float mn = fmaxf(m, mx);
-    const float alpha = exp2f(m - mn);
+    const float alpha = __builtin_amdgcn_exp2f(m - mn);   // v_exp_f32: arguments are <= 0 or -inf here
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float pe = exp2f(sc[r] - mn);
+      const float pe = __builtin_amdgcn_exp2f(sc[r] - mn);
       sc[r] = pe;
       sum += pe;
     }
@@ -434,19 +476,27 @@ __global__ void __launch_bounds__(128) sink_attn_merge_kernel(bf16_t* out, const
 template <int NDB, int NW, int NKC> hipError_t launch_mfma(const SinkAttnArgs& a, hipStream_t s) {
   auto* fn = sink_attn_mfma_kernel<NDB, NW, NKC>;
   const int kp = a.dim + a.vdim + 8, qp = a.dim + 8;
-  const size_t lds = sizeof(bf16_t) * ((size_t)32 * NW * qp + (size_t)MKT * kp) + sizeof(int) * BT_LDS_MAX;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       96 * 1024);
-    if (e != hipSuccess) return e;
-    attr_set = true;
+  const int qpg0 = a.heads / a.kv_heads;
+  const int qr = NW == 1 ? min(32, a.max_q * qpg0 + 1) : 32 * NW;
+  const int nsp = a.ws_o != nullptr ? max(1, a.nsplit) : 1;
+  // block-table entries staged per workgroup: its key range's (else they are read from global memory)
+  const int btc = min(BT_LDS_MAX, (nsp > 1 ? a.chunk / a.block_size + 2 : a.bt_stride) + 1);
+  const size_t lds = sizeof(bf16_t) * ((size_t)qr * qp + (size_t)MKT * kp) + sizeof(int) * btc;
+  if (lds > 150 * 1024) return hipErrorInvalidValue;
+  if (lds > 48 * 1024) {  // only then: the limit is raised per function, and a raised limit is not free
+    static size_t raised = 0;
+    if (lds > raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds);
+      if (e != hipSuccess) return e;
+      raised = lds;
+    }
   }
   const int qpg = a.heads / a.kv_heads;
   const int nsplit = a.ws_o != nullptr ? max(1, a.nsplit) : 1;
   const dim3 grid((unsigned)(((int64_t)a.max_q * qpg + 32 * NW - 1) / (32 * NW)), (unsigned)a.num_seqs,
                   (unsigned)(a.kv_heads * nsplit));
-  hipLaunchKernelGGL(fn, grid, dim3(64 * NW), lds, s, a, kp, qp, a.ws_o, a.ws_ml, nsplit, a.chunk);
+  hipLaunchKernelGGL(fn, grid, dim3(64 * NW), lds, s, a, kp, qp, qr, btc, a.ws_o, a.ws_ml, nsplit, a.chunk);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || nsplit <= 1) return e;
   hipLaunchKernelGGL(sink_attn_merge_kernel, dim3((unsigned)((int64_t)a.heads * a.total_q)), dim3(128), 0, s,

@@ -224,6 +224,27 @@ def gated_delta(qkv32: torch.Tensor, bg: torch.Tensor, gate: torch.Tensor, norm_
 
 
 # ---------------------------------------------------------------------------------------------------- attention
+def _head_major(cache: torch.Tensor, kv_heads: int) -> "_HeadMajorView":
+    return _HeadMajorView(cache, kv_heads)
+
+
+class _HeadMajorView:
+    """Slot-indexed reads and writes (CPU path) of a cache [blocks, block_size, G * (dim + vdim)] whose blocks are
+    laid out head-major inside, [G][block_size][K | V], so that what one key/value head reads from a block is
+    contiguous: item [slots] is [n, G, dim + vdim]."""
+
+    def __init__(self, cache: torch.Tensor, kv_heads: int):
+        nb, bs, w = cache.shape
+        self.v = cache.view(nb, kv_heads, bs, w // kv_heads)
+        self.bs = bs
+
+    def __getitem__(self, slots: torch.Tensor) -> torch.Tensor:
+        return self.v[slots // self.bs, :, slots % self.bs]
+
+    def __setitem__(self, slots: torch.Tensor, rows: torch.Tensor) -> None:
+        self.v[slots // self.bs, :, slots % self.bs] = rows
+
+
 def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Tensor, heads: int, kv_heads: int,
              dim: int, vdim: int, positions: torch.Tensor, slots: torch.Tensor, eps: float,
              q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, rot_dims: int = 0,
@@ -232,8 +253,8 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Ten
     """The step between the q/k/v projection and the attention, one launch: optional RMS norm of q and of k over the
     whole projection (plain weights), optional rotate-half rotary on the first ``rot_dims`` dims of every head (pair
     i, i + rot_dims / 2, angle position * inv_freq[i]), values either divided by their per-head root mean square or
-    blended as (1 - l) v + l v_first; writes the cache row [k | v] at slots[t] (< 0: skipped) and returns q
-    [T, H * dim]."""
+    blended as (1 - l) v + l v_first; writes the token's keys and values into the cache at slots[t] (< 0: skipped;
+    a block's interior is head-major, [G][block_size][k | v]) and returns q [T, H * dim]."""
     T = q.shape[0]
     if q.is_cuda:
         q_out = torch.empty(T, heads * dim, dtype=q.dtype, device=q.device)
@@ -263,8 +284,8 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Ten
         vh = vf.view(T, kv_heads, vdim)
         vf = (vh / torch.sqrt((vh * vh).mean(-1, keepdim=True) + eps)).reshape(T, kv_heads * vdim)
     ok = slots >= 0
-    flat = cache.view(-1, cache.shape[-1])
-    flat[slots[ok]] = torch.cat([kf, vf], 1)[ok].to(cache.dtype)
+    _head_major(cache, kv_heads)[slots[ok]] = torch.cat(
+        [kf.view(T, kv_heads, dim), vf.view(T, kv_heads, vdim)], 2)[ok].to(cache.dtype)
     return qf.to(q.dtype)
 
 
@@ -272,7 +293,7 @@ def sink_attn(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, 
               ctx_lens: torch.Tensor, positions: torch.Tensor, sink: Optional[torch.Tensor],
               bias: Optional[torch.Tensor], max_q: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
               scale: float, impl: int = 0) -> torch.Tensor:
-    """Grouped-query attention over cache rows [k: G * dim | v: G * vdim]. The query at position p sees the cached
+    """Grouped-query attention over the cache that :func:`qkv_prep` writes. The query at position p sees the cached
     positions j <= p with p - j < window (0: all); score (q . k_j) * scale + bias[min(p - j, rows - 1), h]; the
     softmax denominator has one more term exp(sink[h]). Returns [T, H * vdim]. ``impl``: 0 = the matrix-core
     kernel where it applies, 1 = the FMA kernel, 2 = the matrix-core kernel or an error."""
@@ -283,7 +304,7 @@ def sink_attn(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, 
                           dim, vdim, window, scale, impl)
         return out
     bs = cache.shape[1]
-    flat = cache.view(-1, cache.shape[-1]).float()
+    hm = _head_major(cache, kv_heads)
     out = torch.zeros(T, heads, vdim)
     qh = q.float().view(T, heads, dim)
     S = block_tables.shape[0]
@@ -295,9 +316,9 @@ def sink_attn(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, 
             continue
         n_ctx = int(ctx_lens[s])
         j = torch.arange(n_ctx)
-        rows = block_tables[s].long()[j // bs] * bs + j % bs
-        kk = flat[rows, : kv_heads * dim].view(n_ctx, kv_heads, dim).repeat_interleave(rep, 1)
-        vv = flat[rows, kv_heads * dim:].view(n_ctx, kv_heads, vdim).repeat_interleave(rep, 1)
+        rows = hm[block_tables[s].long()[j // bs] * bs + j % bs].float()      # [n_ctx, G, dim + vdim]
+        kk = rows[:, :, :dim].repeat_interleave(rep, 1)
+        vv = rows[:, :, dim:].repeat_interleave(rep, 1)
         for t in range(cu[s], cu[s + 1]):
             n = pos[t] - j
             ok = (n >= 0) & ((n < window) if window > 0 else torch.ones_like(n, dtype=torch.bool))
