@@ -335,27 +335,34 @@ void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTenso
   a.nsplit = 1;
   a.chunk = 0;
   Tensor ws_o, ws_ml;
-  if (die::sink_attn_uses_mfma(a)) {
-    // few row tiles (decode steps): split the keys over workgroups until about 2048 are in flight. The key range is
-    // bounded by the window, else by the block table's width (under a captured graph: the model length; splits
-    // beyond a sequence's keys exit at once)
+  // The key range is bounded by the window, else by the block table's width (under a captured graph: the model
+  // length; splits beyond a sequence's keys exit at once)
+  int64_t bound = block_tables.size(1) * cache.size(1);
+  if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
+  int64_t ns = 1;
+  if (die::sink_attn_uses_decode(a)) {
+    // decode steps: a workgroup per (sequence, key/value head, split); trips of 128 keys, splits until about 1024
+    // workgroups are in flight
+    const int64_t wgs = S * kv_heads;
+    ns = std::min<int64_t>({(int64_t)128, std::max<int64_t>(1, 1024 / std::max<int64_t>(1, wgs)), (bound + 127) / 128});
+    if (ns > 1) a.chunk = (int)((((bound + ns - 1) / ns) + 127) / 128 * 128);
+  } else if (die::sink_attn_uses_mfma(a)) {
+    // few row tiles: split the keys over workgroups until about 2048 are in flight
     const int64_t qpg = heads / kv_heads;
     const int64_t rows_wg = max_q * qpg <= 32 ? 32 : 128;
     const int64_t tiles = S * kv_heads * ((max_q * qpg + rows_wg - 1) / rows_wg);
-    int64_t bound = block_tables.size(1) * cache.size(1);
-    if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
-    const int64_t ns = std::min<int64_t>({(int64_t)16, 2048 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
-    if (ns > 1) {
-      a.chunk = (int)((((bound + ns - 1) / ns) + 31) / 32 * 32);
-      a.nsplit = (int)((bound + a.chunk - 1) / a.chunk);
-      if (a.nsplit > 1) {
-        ws_o = at::empty({a.nsplit, T * heads, vdim}, q.options().dtype(at::kFloat));
-        ws_ml = at::empty({a.nsplit, T * heads, 2}, q.options().dtype(at::kFloat));
-        a.ws_o = ws_o.data_ptr<float>();
-        a.ws_ml = ws_ml.data_ptr<float>();
-      } else {
-        a.nsplit = 1;
-      }
+    ns = std::min<int64_t>({(int64_t)16, 2048 / std::max<int64_t>(1, tiles), (bound + 63) / 64});
+    if (ns > 1) a.chunk = (int)((((bound + ns - 1) / ns) + 31) / 32 * 32);
+  }
+  if (ns > 1) {
+    a.nsplit = (int)((bound + a.chunk - 1) / a.chunk);
+    if (a.nsplit > 1) {
+      ws_o = at::empty({a.nsplit, T * heads, vdim}, q.options().dtype(at::kFloat));
+      ws_ml = at::empty({a.nsplit, T * heads, 2}, q.options().dtype(at::kFloat));
+      a.ws_o = ws_o.data_ptr<float>();
+      a.ws_ml = ws_ml.data_ptr<float>();
+    } else {
+      a.nsplit = 1;
     }
   }
   HIP_OK(die::launch_sink_attn(a, cur_stream()));

@@ -117,7 +117,8 @@ struct SinkAttnArgs {
   int window;             // keys j with 0 <= p - j < window (0: all j <= p)
   float scale;
   bool f32;
-  int impl;               // 0: matrix cores where they apply, else FMA; 1: FMA; 2: matrix cores or fail
+  int impl;               // 0: the decode-step kernel or matrix cores where they apply, else FMA; 1: FMA;
+                          // 2: matrix cores or fail
   // split keys (matrix-core kernel only): nsplit > 1 workgroups per row tile take `chunk` keys each and write
   // unnormalised partial sums to ws_o [nsplit, T * H, vdim] and (running max in log2 units, sum) to
   // ws_ml [nsplit, T * H, 2]; a merge kernel then writes `out`
@@ -127,5 +128,8 @@ struct SinkAttnArgs {
 };
 hipError_t launch_sink_attn(const SinkAttnArgs& a, hipStream_t s);
 bool sink_attn_uses_mfma(const SinkAttnArgs& a);
+// whether launch_sink_attn would run the decode-step kernel (impl 0, one bf16 query token per sequence); it splits
+// the keys in multiples of 128
+bool sink_attn_uses_decode(const SinkAttnArgs& a);
 
 }  // namespace die

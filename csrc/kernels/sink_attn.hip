@@ -451,25 +451,214 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------
+// Decode steps (one query token per sequence) in bf16, dim % 8 == 0 <= 128, vdim % 8 == 0 <= 128, at most 8 query
+// heads per key/value head: no matrix cores and no staging of keys in LDS. A workgroup of 256 threads owns one
+// (sequence, key/value head, split of the keys) and walks its keys 128 at a time:
+//   scores   LK lanes share a key (16 bytes of it each, the query's matching 8 dims in registers), 256 / LK keys
+//            per pass, all passes' loads issued before the first is used; a shuffle reduction per row
+//   softmax  one wave per query row over the 128 scores in LDS (log2 units, running max and sum across trips,
+//            the sink seeds split 0)
+//   values   16 lanes share a value row, 16 keys per pass, loads issued before the softmax; each thread keeps
+//            R x 8 output columns and the 16 key groups are summed through LDS at the end
+// Splits write unnormalised sums + (max, sum) to the workspace and sink_attn_merge_kernel combines them.
+constexpr int DCH = 128;   // keys per trip
+
+template <int R, int LK>
+__global__ void __launch_bounds__(256) sink_attn_decode_kernel(SinkAttnArgs a, float* ws_o, float* ws_ml, int nsplit,
+                                                              int chunk) {
+  constexpr int NG = 256 / LK, NPK = DCH / NG, NPV = DCH / 16;
+  extern __shared__ __attribute__((aligned(16))) float dsm[];
+  float* sc = dsm;                       // [R][DCH] scores, then weights
+  float* ml = sc + R * DCH;              // [R][3]: running max, running sum, this trip's rescale
+  float* red = ml + R * 4;               // [16][R][DV]
+  __shared__ int btl[DCH / 1 + 2];       // block-table entries of the trip (at most one per key)
+  const int z = blockIdx.x, s = blockIdx.y, g = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = a.heads, G = a.kv_heads, QPG = H / G, D = a.dim, DV = a.vdim, roww = D + DV;
+  const int p = (int)a.positions[s];
+  const int ctx = a.ctx_lens[s];
+  int jlo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  int jhi = min(p, ctx - 1);
+  if (nsplit > 1) {
+    jlo += z * chunk;
+    jhi = min(jhi, jlo + chunk - 1);
+  }
+  const int64_t wrows = (int64_t)a.total_q * H;
+  if (jlo > jhi) {   // an empty split: it only reports that it holds nothing
+    if (nsplit > 1 && tid < QPG) {
+      const int64_t orow = (int64_t)s * H + g * QPG + tid;
+      ws_ml[((int64_t)z * wrows + orow) * 2] = -1e30f;
+      ws_ml[((int64_t)z * wrows + orow) * 2 + 1] = 0.f;
+    }
+    return;
+  }
+  constexpr float LOG2E = 1.4426950408889634f;
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+  const bf16_t* qg = reinterpret_cast<const bf16_t*>(a.q);
+  const int* bt = a.block_tables + (int64_t)s * a.bt_stride;
+  const int kl = tid % LK, kg = tid / LK;      // score phase: my 8 dims of the key, my key group
+  const int vl = tid & 15, vg = tid >> 4;      // value phase: my 8 columns, my key group
+  float qf[R][8];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (r < QPG && 8 * kl < D) unpack8(*reinterpret_cast<const uint4*>(qg + ((int64_t)s * H + g * QPG + r) * D + 8 * kl), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[r][e] = f[e] * (a.scale * LOG2E);
+  }
+  if (tid < R) {
+    const bool has_sink = a.sink != nullptr && tid < QPG && z == 0;
+    ml[tid * 4] = has_sink ? a.sink[g * QPG + tid] * LOG2E : -1e30f;
+    ml[tid * 4 + 1] = has_sink ? 1.0f : 0.0f;
+  }
+  float acc[R][8];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+
+  for (int j0 = jlo; j0 <= jhi; j0 += DCH) {
+    const int b_lo = j0 / a.block_size;
+    __syncthreads();   // the previous trip's weights and block-table entries are no longer read
+    {
+      const int nb = min(jhi, j0 + DCH - 1) / a.block_size - b_lo + 1;
+      if (tid < nb) btl[tid] = bt[b_lo + tid];
+    }
+    __syncthreads();
+    uint4 kq[NPK], vq[NPV];
+#pragma unroll
+    for (int u = 0; u < NPK; ++u) {
+      const int j = j0 + u * NG + kg;
+      kq[u] = make_uint4(0, 0, 0, 0);
+      if (j <= jhi && 8 * kl < D) {
+        const int jb = j / a.block_size;
+        kq[u] = *reinterpret_cast<const uint4*>(
+            cache + (((int64_t)btl[jb - b_lo] * G + g) * a.block_size + (j - jb * a.block_size)) * roww + 8 * kl);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NPV; ++u) {
+      const int j = j0 + u * 16 + vg;
+      vq[u] = make_uint4(0, 0, 0, 0);
+      if (j <= jhi && 8 * vl < DV) {
+        const int jb = j / a.block_size;
+        vq[u] = *reinterpret_cast<const uint4*>(
+            cache + (((int64_t)btl[jb - b_lo] * G + g) * a.block_size + (j - jb * a.block_size)) * roww + D + 8 * vl);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NPK; ++u) {
+      float f[8];
+      unpack8(kq[u], f);
+      const int jj = u * NG + kg, j = j0 + jj;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d += qf[r][e] * f[e];
+#pragma unroll
+        for (int off = 1; off < LK; off <<= 1) d += __shfl_xor(d, off, 64);
+        if (kl == 0) {
+          const int n = p - j;
+          const bool valid = r < QPG && j <= jhi && n >= 0;
+          if (valid && a.bias != nullptr) d += a.bias[(int64_t)min(n, a.bias_rows - 1) * H + g * QPG + r] * LOG2E;
+          sc[r * DCH + jj] = valid ? d : -INFINITY;
+        }
+      }
+    }
+    __syncthreads();
+    for (int r = wave; r < R; r += 4) {
+      const float v0 = sc[r * DCH + lane], v1 = sc[r * DCH + 64 + lane];
+      const float m0 = ml[r * 4], l0 = ml[r * 4 + 1];
+      const float mn = fmaxf(m0, wave_max(fmaxf(v0, v1)));
+      const float p0 = __builtin_amdgcn_exp2f(v0 - mn), p1 = __builtin_amdgcn_exp2f(v1 - mn);
+      const float alpha = __builtin_amdgcn_exp2f(m0 - mn);
+      const float sum = wave_sum(p0 + p1);
+      sc[r * DCH + lane] = p0;
+      sc[r * DCH + 64 + lane] = p1;
+      if (lane == 0) {
+        ml[r * 4] = mn;
+        ml[r * 4 + 1] = l0 * alpha + sum;
+        ml[r * 4 + 2] = alpha;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float alpha = ml[r * 4 + 2];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[r][e] *= alpha;
+    }
+#pragma unroll
+    for (int u = 0; u < NPV; ++u) {
+      float f[8];
+      unpack8(vq[u], f);
+      const int jj = u * 16 + vg;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float pw = sc[r * DCH + jj];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][e] += pw * f[e];
+      }
+    }
+  }
+  // sum the 16 key groups
+  if (8 * vl < DV) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float* dst = red + ((int64_t)vg * R + r) * DV + 8 * vl;
+      *reinterpret_cast<float4*>(dst) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+      *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < QPG * DV; idx += 256) {
+    const int r = idx / DV, c = idx % DV;
+    float o = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) o += red[((int64_t)k * R + r) * DV + c];
+    const int64_t orow = (int64_t)s * H + g * QPG + r;
+    if (nsplit > 1) {
+      ws_o[((int64_t)z * wrows + orow) * DV + c] = o;
+      if (c == 0) {
+        ws_ml[((int64_t)z * wrows + orow) * 2] = ml[r * 4];
+        ws_ml[((int64_t)z * wrows + orow) * 2 + 1] = ml[r * 4 + 1];
+      }
+    } else {
+      const float l = ml[r * 4 + 1];
+      reinterpret_cast<bf16_t*>(a.out)[orow * DV + c] = f2bf(l > 0.f ? o / l : 0.f);
+    }
+  }
+}
+
 // out[row] = sum_z O_z 2^(m_z - m*) / sum_z l_z 2^(m_z - m*), m* = max_z m_z (running maxima in log2 units).
 __global__ void __launch_bounds__(128) sink_attn_merge_kernel(bf16_t* out, const float* ws_o, const float* ws_ml,
                                                               int nsplit, int64_t rows, int DV) {
+  __shared__ float wz[128];   // a split's weight 2^(m_z - m*) / sum (nsplit <= 128)
   const int64_t row = blockIdx.x;
-  float mstar = -1e30f;
-  for (int z = 0; z < nsplit; ++z) mstar = fmaxf(mstar, ws_ml[((int64_t)z * rows + row) * 2]);
-  float lsum = 0.f;
-  for (int z = 0; z < nsplit; ++z) {
-    const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
-    if (lz > 0.f) lsum += lz * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
-  }
-  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  const int z = threadIdx.x;
+  const float mz = z < nsplit ? ws_ml[((int64_t)z * rows + row) * 2] : -1e30f;
+  const float lz = z < nsplit ? ws_ml[((int64_t)z * rows + row) * 2 + 1] : 0.f;
+  float mstar = wave_max(mz);
+  __shared__ float red2[4];
+  if ((threadIdx.x & 63) == 0) red2[threadIdx.x >> 6] = mstar;
+  __syncthreads();
+  mstar = fmaxf(red2[0], red2[1]);
+  const float w = lz > 0.f ? exp2f(mz - mstar) : 0.f;
+  float lsum = wave_sum(lz * w);
+  if ((threadIdx.x & 63) == 0) red2[2 + (threadIdx.x >> 6)] = lsum;
+  __syncthreads();
+  lsum = red2[2] + red2[3];
+  wz[z] = lsum > 0.f ? w / lsum : 0.f;
+  __syncthreads();
   for (int c = threadIdx.x; c < DV; c += 128) {
     float acc = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-      const float lz = ws_ml[((int64_t)z * rows + row) * 2 + 1];
-      if (lz > 0.f) acc += ws_o[((int64_t)z * rows + row) * DV + c] * exp2f(ws_ml[((int64_t)z * rows + row) * 2] - mstar);
+    for (int k = 0; k < nsplit; ++k) {
+      const float wk = wz[k];
+      if (wk != 0.f) acc += ws_o[((int64_t)k * rows + row) * DV + c] * wk;
     }
-    out[row * DV + c] = f2bf(acc * inv);
+    out[row * DV + c] = f2bf(acc);
   }
 }
 
@@ -518,6 +707,41 @@ template <int NW> hipError_t launch_mfma_nw(const SinkAttnArgs& a, hipStream_t s
   return a.dim <= 64 ? launch_mfma_ndb<NW, 8>(a, s) : launch_mfma_ndb<NW, 16>(a, s);
 }
 
+template <int R, int LK> hipError_t launch_decode_one(const SinkAttnArgs& a, hipStream_t s) {
+  auto* fn = sink_attn_decode_kernel<R, LK>;
+  const size_t lds = sizeof(float) * ((size_t)R * DCH + (size_t)R * 4 + (size_t)16 * R * a.vdim);
+  if (lds > 48 * 1024) {
+    static size_t raised = 0;
+    if (lds > raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds);
+      if (e != hipSuccess) return e;
+      raised = lds;
+    }
+  }
+  const int nsplit = a.ws_o != nullptr ? max(1, a.nsplit) : 1;
+  hipLaunchKernelGGL(fn, dim3(nsplit, a.num_seqs, a.kv_heads), dim3(256), lds, s, a, a.ws_o, a.ws_ml, nsplit, a.chunk);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || nsplit <= 1) return e;
+  hipLaunchKernelGGL(sink_attn_merge_kernel, dim3((unsigned)((int64_t)a.heads * a.total_q)), dim3(128), 0, s,
+                     reinterpret_cast<bf16_t*>(a.out), a.ws_o, a.ws_ml, nsplit, (int64_t)a.heads * a.total_q, a.vdim);
+  return hipGetLastError();
+}
+
+template <int LK> hipError_t launch_decode_r(const SinkAttnArgs& a, hipStream_t s) {
+  const int qpg = a.heads / a.kv_heads;
+  if (qpg <= 1) return launch_decode_one<1, LK>(a, s);
+  if (qpg <= 2) return launch_decode_one<2, LK>(a, s);
+  if (qpg <= 4) return launch_decode_one<4, LK>(a, s);
+  return launch_decode_one<8, LK>(a, s);
+}
+
+inline bool decode_ok(const SinkAttnArgs& a) {
+  return !a.f32 && a.cu_q == nullptr && a.max_q == 1 && a.heads / a.kv_heads <= 8 && a.dim % 8 == 0 && a.dim <= 128 &&
+         a.vdim % 8 == 0 && a.vdim <= 128 && (reinterpret_cast<uintptr_t>(a.q) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0 && (a.nsplit <= 1 || a.nsplit <= 128);
+}
+
 inline bool mfma_ok(const SinkAttnArgs& a) {
   return !a.f32 && a.dim % 16 == 0 && a.dim <= 128 && a.vdim % 32 == 0 && a.vdim <= 128 &&
          (reinterpret_cast<uintptr_t>(a.q) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0 &&
@@ -527,12 +751,14 @@ inline bool mfma_ok(const SinkAttnArgs& a) {
 }  // namespace
 
 bool sink_attn_uses_mfma(const SinkAttnArgs& a) { return a.impl != 1 && mfma_ok(a); }
+bool sink_attn_uses_decode(const SinkAttnArgs& a) { return a.impl == 0 && decode_ok(a); }
 
 hipError_t launch_sink_attn(const SinkAttnArgs& a, hipStream_t s) {
   if (a.num_seqs == 0 || a.total_q == 0) return hipSuccess;
   if (a.heads < 1 || a.kv_heads < 1 || a.heads % a.kv_heads != 0 || a.dim < 1 || a.dim > 512 || a.vdim < 1 ||
       a.vdim > 256 || a.block_size < 1 || a.max_q < 1 || (a.bias != nullptr && a.bias_rows < 1))
     return hipErrorInvalidValue;
+  if (sink_attn_uses_decode(a)) return a.dim <= 64 ? launch_decode_r<8>(a, s) : launch_decode_r<16>(a, s);
   if (sink_attn_uses_mfma(a)) {
     const int qpg = a.heads / a.kv_heads;
     return a.max_q * qpg <= 32 ? launch_mfma_nw<1>(a, s) : launch_mfma_nw<4>(a, s);
