@@ -341,10 +341,10 @@ void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTenso
   if (window > 0) bound = std::min<int64_t>(bound, window + max_q);
   int64_t ns = 1;
   if (die::sink_attn_uses_decode(a)) {
-    // decode steps: a workgroup per (sequence, key/value head, split); trips of 128 keys, splits until about 1024
+    // decode steps: a workgroup per (sequence, key/value head, split); trips of 128 keys, splits until about 2048
     // workgroups are in flight
     const int64_t wgs = S * kv_heads;
-    ns = std::min<int64_t>({(int64_t)128, std::max<int64_t>(1, 1024 / std::max<int64_t>(1, wgs)), (bound + 127) / 128});
+    ns = std::min<int64_t>({(int64_t)128, std::max<int64_t>(1, 2048 / std::max<int64_t>(1, wgs)), (bound + 127) / 128});
     if (ns > 1) a.chunk = (int)((((bound + ns - 1) / ns) + 127) / 128 * 128);
   } else if (die::sink_attn_uses_mfma(a)) {
     // few row tiles: split the keys over workgroups until about 2048 are in flight

@@ -239,44 +239,52 @@ __global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void
   __shared__ float red[NT / 64];
   const int64_t r = blockIdx.x;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  // bf16 rows of a multiple of 8 columns, up to 8 * KEEP * NT wide: 16-byte accesses, the row kept in registers
-  constexpr int KEEP = 4;
-  if (!f32 && n % 8 == 0 && n <= 8 * KEEP * NT && zstride % 8 == 0 && aligned16(z) && aligned16(out)) {
+  // bf16 rows of a multiple of 8 columns: 16-byte accesses; the first KEEP trips stay in registers between the two
+  // passes (rows up to 8 * KEEP * NT wide are read once), wider rows re-read the rest
+  constexpr int KEEP = 8;
+  if (!f32 && n % 8 == 0 && zstride % 8 == 0 && aligned16(z) && aligned16(out)) {
     const uint4* zr = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(z) + r * zstride);
+    const int n8 = n / 8;
     uint4 keep[KEEP];
+    auto sums = [&](const uint4& v) {
+      float f[8];
+      unpack8(v, f);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float v2 = f[q] * f[q];
+        s2 += v2;
+        s4 += v2 * v2;
+        s6 += v2 * v2 * v2;
+      }
+    };
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
       const int c8 = it * NT + threadIdx.x;
-      if (c8 < n / 8) {
+      if (c8 < n8) {
         keep[it] = zr[c8];
-        float f[8];
-        unpack8(keep[it], f);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const float v2 = f[q] * f[q];
-          s2 += v2;
-          s4 += v2 * v2;
-          s6 += v2 * v2 * v2;
-        }
+        sums(keep[it]);
       }
     }
+    for (int c8 = KEEP * NT + threadIdx.x; c8 < n8; c8 += NT) sums(zr[c8]);
     s2 = block_sum<NT>(s2, red);
     s4 = block_sum<NT>(s4, red);
     s6 = block_sum<NT>(s6, red);
     const float r1 = coef[0] / sqrtf(s2 / (float)n + eps), r2 = coef[1] / sqrtf(s4 / (float)n + eps),
                 r3 = coef[2] / sqrtf(s6 / (float)n + eps), c3 = coef[3];
     uint4* orow = reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(out) + r * n);
+    auto apply = [&](const uint4& v) -> uint4 {
+      float f[8];
+      unpack8(v, f);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) f[q] = f[q] * r1 + f[q] * f[q] * r2 + f[q] * f[q] * f[q] * r3 + c3;
+      return pack8(f);
+    };
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
       const int c8 = it * NT + threadIdx.x;
-      if (c8 < n / 8) {
-        float f[8];
-        unpack8(keep[it], f);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) f[q] = f[q] * r1 + f[q] * f[q] * r2 + f[q] * f[q] * f[q] * r3 + c3;
-        orow[c8] = pack8(f);
-      }
+      if (c8 < n8) orow[c8] = apply(keep[it]);
     }
+    for (int c8 = KEEP * NT + threadIdx.x; c8 < n8; c8 += NT) orow[c8] = apply(zr[c8]);
     return;
   }
   for (int c = threadIdx.x; c < n; c += NT) {
