@@ -544,6 +544,41 @@ def test_unequal_batch_equals_each_alone_and_slots_are_reused(tmp_path, device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_medium_model_long_prompts_in_mixed_steps(tmp_path, device, dtype):
+    """A model at the scale of a real small one (width 192, head dims 48 - 96, window 100, 24 distance buckets,
+    attention first): prompts several windows and pages long, run as a whole, in portions, token by token and
+    beside each other with slots reused. bf16 on the GPU takes the matrix-core kernel where the shapes allow
+    (dim 64 / vdim 96, dim 80), the FMA kernel elsewhere (vdim 48) and the decode-step kernel for single tokens."""
+    _need(device)
+    att = orc.attn_cfg(heads=6, kv_heads=2, dim=64, vdim=96, window=100, bias_max=70.0)
+    par = orc.parallel_cfg(heads=6, kv_heads=3, dim=80, vdim=48, rot_dims=40, rot_base=5000.0, r_heads=6, r_kv_heads=2,
+                           r_dim=48, r_vdim=32, conv=3, left_scale=1.2, right_scale=0.5)
+    cfg = orc.make_config([("attention", att, 320), ("parallel", par, None), ("attention", att, 256)], width=192,
+                          vocab=211, streams=2, buckets=97)
+    wts = orc.make_weights(cfg, seed=33, rel_rows=24)
+    eng = make_engine(tmp_path, cfg, wts, device, dtype, max_tokens=448, max_seqs=3, block_size=32)
+    a, b, c = tokens_for(cfg, 230, 1), tokens_for(cfg, 150, 2), tokens_for(cfg, 40, 3)
+    at = {"a": 0, "b": 0, "c": 0}
+    toks = {"a": a, "b": b, "c": c}
+
+    def ent(k, n, want=None):
+        lo = at[k]
+        hi = min(lo + n, len(toks[k]))
+        at[k] = hi
+        w = list(range(hi - lo)) if want is None else want
+        return (k, toks[k][lo:hi], w, hi == len(toks[k]))
+
+    steps = [[ent("a", 130)], [ent("a", 1), ent("b", 97)], [ent("a", 1), ent("b", 2)], [ent("a", 1), ent("b", 1)],
+             [ent("a", 64), ent("b", 50), ent("c", 33)], [ent("a", 33), ent("c", 7)]]
+    got = replay(eng, steps)
+    for k in ("a", "b", "c"):
+        assert at[k] == len(toks[k])
+        check_against_oracle(got[k], wts, cfg, toks[k], TOL[dtype])
+    assert eng.blocks.num_available() == eng.blocks.num_blocks
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_window_edges_sink_state_and_far_keys_show_in_logits(tmp_path, device):
     """The engine agrees with the oracle where the oracle itself is sensitive: a window one token longer or shorter,
     no sink, no bias, a decay of one, a convolution without its oldest tap and a far key all move the oracle's
