@@ -71,7 +71,7 @@ def fekolorn_arch(z):
     left = SinkAttnSpec(z["heads"], z["kv_heads"], z["dim"], z["vdim"], scale, rot_dims=z["dim"] // 2, v_unit=True)
     right = GatedDeltaSpec(z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["conv"])
     att = SinkAttnSpec(z["heads"], z["kv_heads"], z["dim"], z["vdim"], scale, window=z["window"], qk_norm=True,
-                       v_mix=True, bias_max=float(z["window"]))
+                       v_mix=True, bias_max=128.0)
     mlp = PolyMlpSpec(z["ff"])
     layers = []
     for i in range(z["layers"]):
@@ -109,7 +109,7 @@ def kernels(z, a, size):
 
     cache = (torch.randn(nb, bs, G * (D + DV), device=dev) * 0.5).to(bf)
     sink = torch.zeros(H, device=dev)
-    bias = torch.zeros(L + 1, H, device=dev)
+    bias = torch.zeros(130, H, device=dev)   # distances up to 128 have their own bias, the rest share one
     scale = 1.0 / math.sqrt(D)
     for mode, T, pos, cuq, mq in (("prefill", S * L, torch.arange(L, device=dev).repeat(S), cu, L),
                                   ("decode", S, torch.full((S,), L - 1, device=dev), None, 1)):
