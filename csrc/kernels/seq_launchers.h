@@ -26,11 +26,12 @@ struct RaggedRows {
 
 // streams[t, s, :] (fp32, s < S) = embed[ids[t]] * scale + bigram[row(t)] for all s. row(t) = buckets at
 // position 0, else (prev * mul_prev + ids[t] * mul_cur) mod buckets, prev = the sequence's previous token (the
-// row before, or prev_tok[slot] for the first row of the step). bigram == nullptr: no such term.
+// row before, or prev_tok[slot] for the first row of the step). bigram == nullptr: no such term. A step with one row
+// per sequence (cu_q == nullptr) also stores the row's token as the slot's new previous token.
 hipError_t launch_embed_hash(float* streams, int S, int W, const void* embed, const void* bigram, bool f32,
-                             const int64_t* ids, RaggedRows r, const int64_t* prev_tok, float scale, int64_t buckets,
+                             const int64_t* ids, RaggedRows r, int64_t* prev_tok, float scale, int64_t buckets,
                              int64_t mul_prev, int64_t mul_cur, hipStream_t s);
-// prev_tok[slot(s)] = the last token of sequence s in this step
+// prev_tok[slot(s)] = the last token of sequence s in this step (nothing to do when cu_q == nullptr, see above)
 hipError_t launch_store_last_token(int64_t* prev_tok, const int64_t* ids, RaggedRows r, hipStream_t s);
 
 struct StreamMixArgs {
@@ -64,11 +65,12 @@ struct DeltaShape {
 // Per row: the short causal convolution (+ SiLU) of the C = [q | k | v] channels of x, with the taps - 1 inputs
 // before the step taken from conv_state [slots, taps - 1, C] (fp32, the most recent last); q and k heads made
 // unit vectors (q also times dim^-1/2); beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)).
-// Writes qkv32 [T, C] and bg [T, 2 * heads] = [beta | g], both fp32.
+// Writes qkv32 [T, C] and bg [T, 2 * heads] = [beta | g], both fp32. A step with one row per sequence
+// (cu_q == nullptr) also moves the row's input into conv_state.
 hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void* b, const void* a, int64_t xstride,
-                             bool f32, const float* conv_w, const float* conv_state, const float* A_log,
+                             bool f32, const float* conv_w, float* conv_state, const float* A_log,
                              const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s);
-// conv_state[slot(s)] = the last taps - 1 inputs of sequence s after this step
+// conv_state[slot(s)] = the last taps - 1 inputs of sequence s after this step (nothing to do when cu_q == nullptr)
 hipError_t launch_conv_state_update(float* conv_state, const void* x, int64_t xstride, bool f32, DeltaShape sh,
                                     RaggedRows r, hipStream_t s);
 // Per (sequence, head), token by token: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with

@@ -69,7 +69,7 @@ __device__ __forceinline__ int seq_of_row(const int* cu_q, int num_seqs, int row
 
 __global__ void __launch_bounds__(NT) embed_hash_kernel(float* streams, int S, int W, const void* embed,
                                                        const void* bigram, bool f32, const int64_t* ids,
-                                                       RaggedRows r, const int64_t* prev_tok, float scale,
+                                                       RaggedRows r, int64_t* prev_tok, float scale,
                                                        int64_t buckets, int64_t mul_prev, int64_t mul_cur) {
   const int row = blockIdx.x;
   const int64_t tok = ids[row];
@@ -83,6 +83,11 @@ __global__ void __launch_bounds__(NT) embed_hash_kernel(float* streams, int S, i
       const int first = r.cu_q ? r.cu_q[s] : s;
       const int64_t prev = row > first ? ids[row - 1] : prev_tok[r.state_slots[s]];
       brow = (prev * mul_prev + tok * mul_cur) % buckets;
+    }
+    if (r.cu_q == nullptr) {
+      // one row per sequence: this workgroup is the slot's only reader, so it also stores the new last token
+      __syncthreads();
+      if (threadIdx.x == 0) prev_tok[r.state_slots[row]] = tok;
     }
   }
   float* out = streams + (int64_t)row * S * W;
@@ -308,7 +313,7 @@ __global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void
 // ------------------------------------------------------------------------------------------ gated delta rule
 __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg, const void* x, const void* b,
                                                        const void* a, int64_t xstride, bool f32, const float* conv_w,
-                                                       const float* conv_state, const float* A_log,
+                                                       float* conv_state, const float* A_log,
                                                        const float* dt_bias, DeltaShape sh, RaggedRows r) {
   extern __shared__ float vals[];  // [C]
   const int row = blockIdx.x;
@@ -317,7 +322,7 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
   const int i = row - first;
   const int64_t p = r.positions[row];
   const int C = sh.channels(), taps = sh.taps;
-  const float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
+  float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
   for (int c = threadIdx.x; c < C; c += NT) {
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
@@ -328,6 +333,12 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
       acc += conv_w[(int64_t)c * taps + j] * xv;
     }
     vals[c] = rnd(siluf(rnd(acc, f32)), f32);
+    if (r.cu_q == nullptr) {
+      // one row per sequence: this thread is the only reader of its channel's tail, so it shifts it here
+      for (int k = 0; k + 1 < taps - 1; ++k)
+        st[(int64_t)k * C + c] = p - (taps - 2 - k) >= 0 ? st[(int64_t)(k + 1) * C + c] : 0.f;
+      if (taps > 1) st[(int64_t)(taps - 2) * C + c] = ldv(x, (int64_t)row * xstride + c, f32);
+    }
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -578,7 +589,7 @@ bool rows_ok(const RaggedRows& r) { return r.positions != nullptr && r.state_slo
 }  // namespace
 
 hipError_t launch_embed_hash(float* streams, int S, int W, const void* embed, const void* bigram, bool f32,
-                             const int64_t* ids, RaggedRows r, const int64_t* prev_tok, float scale, int64_t buckets,
+                             const int64_t* ids, RaggedRows r, int64_t* prev_tok, float scale, int64_t buckets,
                              int64_t mul_prev, int64_t mul_cur, hipStream_t s) {
   if (r.total_rows == 0) return hipSuccess;
   if (S < 1 || W < 1 || (bigram != nullptr && (buckets < 1 || prev_tok == nullptr || !rows_ok(r))))
@@ -589,7 +600,7 @@ hipError_t launch_embed_hash(float* streams, int S, int W, const void* embed, co
 }
 
 hipError_t launch_store_last_token(int64_t* prev_tok, const int64_t* ids, RaggedRows r, hipStream_t s) {
-  if (r.num_seqs == 0) return hipSuccess;
+  if (r.num_seqs == 0 || r.cu_q == nullptr) return hipSuccess;  // one row per sequence: embed_hash stored it
   if (!rows_ok(r)) return hipErrorInvalidValue;
   hipLaunchKernelGGL(store_last_token_kernel, dim3((r.num_seqs + 63) / 64), dim3(64), 0, s, prev_tok, ids, r);
   return hipGetLastError();
@@ -616,7 +627,7 @@ static bool delta_ok(const DeltaShape& sh) {
 }
 
 hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void* b, const void* a, int64_t xstride,
-                             bool f32, const float* conv_w, const float* conv_state, const float* A_log,
+                             bool f32, const float* conv_w, float* conv_state, const float* A_log,
                              const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s) {
   if (r.total_rows == 0) return hipSuccess;
   if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
@@ -634,7 +645,7 @@ hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void*
 
 hipError_t launch_conv_state_update(float* conv_state, const void* x, int64_t xstride, bool f32, DeltaShape sh,
                                     RaggedRows r, hipStream_t s) {
-  if (r.num_seqs == 0 || sh.taps <= 1) return hipSuccess;
+  if (r.num_seqs == 0 || sh.taps <= 1 || r.cu_q == nullptr) return hipSuccess;  // one row each: delta_prep did it
   if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
   hipLaunchKernelGGL(conv_state_update_kernel, dim3((sh.channels() + NT - 1) / NT, r.num_seqs), dim3(NT), 0, s,
                      conv_state, x, xstride, f32, sh, r);

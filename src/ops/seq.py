@@ -73,7 +73,8 @@ def embed_hash(ids: torch.Tensor, embed: torch.Tensor, bigram: Optional[torch.Te
                prev_tok: torch.Tensor, scale: float, buckets: int, mul_prev: int, mul_cur: int,
                streams: int) -> torch.Tensor:
     """fp32 [T, streams, W]: embed[id] * scale + bigram[(prev * mul_prev + id * mul_cur) mod buckets] (row
-    ``buckets`` at position 0), copied into every stream."""
+    ``buckets`` at position 0), copied into every stream. On the GPU a step with one row per sequence also stores
+    the row's token as the new previous token (:func:`store_last_token` then has nothing left to do)."""
     T, W = ids.shape[0], embed.shape[1]
     out = torch.empty(T, streams, W, dtype=torch.float32, device=ids.device)
     if ids.is_cuda:
@@ -98,7 +99,8 @@ def embed_hash(ids: torch.Tensor, embed: torch.Tensor, bigram: Optional[torch.Te
 
 def store_last_token(prev_tok: torch.Tensor, ids: torch.Tensor, rag: Ragged) -> None:
     if ids.is_cuda:
-        _kern().store_last_token(prev_tok, ids, rag.positions, rag.cu_q, rag.state_slots)
+        if rag.cu_q is not None:   # one row per sequence: embed_hash stored it
+            _kern().store_last_token(prev_tok, ids, rag.positions, rag.cu_q, rag.state_slots)
         return
     for q0, n, slot in rag.spans(ids.shape[0]):
         prev_tok[slot] = ids[q0 + n - 1]
@@ -151,7 +153,8 @@ def delta_prep(x: torch.Tensor, b: torch.Tensor, a: torch.Tensor, conv_w: torch.
     """x [T, C = 2 G dim + H vdim] = [q | k | v] channels: causal convolution over the sequence's last ``taps``
     inputs (those before the step from conv_state [slots, taps - 1, C]) + SiLU; q and k heads to unit length
     (q also times dim^-1/2). Returns (qkv32 [T, C] fp32, bg [T, 2 H] fp32 = [sigmoid(b) | exp(-exp(A_log) *
-    softplus(a + dt_bias))])."""
+    softplus(a + dt_bias))]). On the GPU a step with one row per sequence also moves the row's input into
+    conv_state (:func:`conv_state_update` then has nothing left to do)."""
     T, C = x.shape
     taps = conv_w.shape[1]
     qkv32 = torch.empty(T, C, dtype=torch.float32, device=x.device)
@@ -185,7 +188,9 @@ def conv_state_update(conv_state: torch.Tensor, x: torch.Tensor, heads: int, kv_
     if conv_state.shape[1] == 0:
         return
     if x.is_cuda:
-        _kern().conv_state_update(conv_state, x, heads, kv_heads, dim, vdim, rag.positions, rag.cu_q, rag.state_slots)
+        if rag.cu_q is not None:   # one row per sequence: delta_prep moved it
+            _kern().conv_state_update(conv_state, x, heads, kv_heads, dim, vdim, rag.positions, rag.cu_q,
+                                      rag.state_slots)
         return
     k = conv_state.shape[1]
     pos = rag.positions.tolist()
