@@ -274,7 +274,8 @@ def _delta_weights(H, G, d, dv, taps, W, seed):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("shape", [(2, 1, 8, 16, 3), (4, 4, 5, 7, 4), (3, 1, 40, 70, 1), (1, 1, 64, 128, 2)])
+@pytest.mark.parametrize("shape", [(2, 1, 8, 16, 3), (4, 4, 5, 7, 4), (3, 1, 40, 70, 1), (1, 1, 64, 128, 2),
+                                   (2, 1, 128, 128, 4), (1, 1, 200, 256, 2)])
 def test_gated_delta_rule_in_portions_and_slots(device, shape):
     """The recurrence with its convolution, cut into portions (down to one token), two sequences sharing steps, in
     slots that held another sequence before."""
@@ -326,7 +327,7 @@ def _paged(device, dtype, n_blocks, bs, width, seed):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", ["rotary", "biased", "wide", "mc_rotary", "mc_biased"])
+@pytest.mark.parametrize("case", ["rotary", "biased", "wide", "mc_rotary", "mc_biased", "served_rotary", "served_biased"])
 def test_attention_ops_with_standout_keys(device, dtype, case):
     """qkv_prep + sink_attn over scattered pages, prompt portion and single decode rows: one key far back, one on a
     page border, and the keys just inside and just outside the window are made to stand out (their scores lead by
@@ -343,6 +344,10 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
         H, G, d, dv, window, rot, bias_max = 8, 2, 80, 32, 0, 48, 0
     elif case == "mc_biased":
         H, G, d, dv, window, rot, bias_max = 6, 2, 32, 96, 37, 0, 15.0
+    elif case == "served_rotary":  # default dispatch at a served shape: 8 query heads on one key/value head
+        H, G, d, dv, window, rot, bias_max = 8, 1, 128, 128, 0, 64, 0
+    elif case == "served_biased":  # default dispatch, one query head per key/value head
+        H, G, d, dv, window, rot, bias_max = 2, 2, 64, 32, 50, 0, 15.0
     else:
         H, G, d, dv, window, rot, bias_max = 2, 1, 96, 160, 40, 0, 0
     impl = 2 if case.startswith("mc_") and dtype == torch.bfloat16 and device != "cpu" else 0
