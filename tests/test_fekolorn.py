@@ -757,3 +757,49 @@ def test_generation_with_decode_graphs(tmp_path):
     got = replay(eng, cut("z", prompts[1] + outs[1], [len(prompts[1])]))["z"]
     check_against_oracle(got, wts, cfg, prompts[1] + outs[1], TOL[torch.bfloat16])
     assert eng.blocks.num_available() == eng.blocks.num_blocks
+
+
+def test_worker_serves_a_fekolorn_checkpoint(tmp_path):
+    """The serving path end to end on the CPU: client -> coordinator -> worker -> LLMBackend -> from_pretrained
+    (the registry picks FekolornLM from config.json) -> continuous-batching engine with state slots -> sampled token
+    ids, which are the oracle's greedy continuation of each prompt. More prompts than sequence slots."""
+    import asyncio
+
+    from src.client import InferenceClient
+    from src.config import ModelConfig
+    from src.coordinator import Coordinator
+    from src.worker import Worker
+
+    cfg = std_config(vocab=300)
+    wts = orc.make_weights(cfg, seed=22)
+    path = str(tmp_path / "served")
+    save_checkpoint(path, cfg, wts)
+    mc = ModelConfig(model_name="fk", model_path=path, arch="llama", max_batch_size=2, max_model_len=128,
+                     max_num_batched_tokens=128, num_kv_blocks=64, use_cuda_graph=False, max_latency_ms=1.0,
+                     overrides={"device": "cpu"})
+
+    async def main():
+        w = Worker("w0", host="127.0.0.1", install_signal_handlers=False)
+        assert w.load_model(mc)
+        wport = await w.start()
+        coord = Coordinator(port=0, max_batch_size=4, max_latency_ms=2)
+        cport = await coord.start()
+        await coord.add_static_worker(f"127.0.0.1:{wport}")
+        c = InferenceClient(f"127.0.0.1:{cport}")
+        prompts = [tokens_for(cfg, n, 40 + n) for n in (4, 19, 11, 7)]
+        rs = await asyncio.wait_for(asyncio.gather(*(c.infer("fk", {"prompt_token_ids": p, "max_tokens": 6,
+                                                                    "ignore_eos": True}) for p in prompts)), 120)
+        c.close()
+        await coord.stop()
+        await w.shutdown()
+        return prompts, rs
+
+    prompts, rs = asyncio.run(main())
+    assert all(r["success"] for r in rs), rs
+    for p, r in zip(prompts, rs):
+        out = r["outputs"]["token_ids"]
+        assert len(out) == 6
+        lg = orc.forward(p + out, wts, cfg)
+        for i, tok in enumerate(out):
+            row = lg[len(p) + i - 1]
+            assert float(row.max() - row[tok]) <= 0.05 * float(row.max() - row.min())
