@@ -159,8 +159,8 @@ die::DeltaShape delta_shape(int64_t heads, int64_t kv_heads, int64_t dim, int64_
 }
 
 // x [T, C], b [T, heads], a [T, heads]: column slices of ONE projection output (same row stride)
-void delta_prep(Tensor qkv32, Tensor bg, Tensor x, Tensor b, Tensor a, Tensor conv_w, Tensor conv_state, Tensor A_log,
-                Tensor dt_bias, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, Tensor positions,
+void delta_prep(Tensor qkv32, Tensor bg, Tensor x, Tensor b, Tensor a, Tensor conv_w, OptTensor conv_wt,
+                Tensor conv_state, Tensor A_log, Tensor dt_bias, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, Tensor positions,
                 OptTensor cu_q, Tensor state_slots) {
   TORCH_CHECK(conv_w.dim() == 2, "conv_w [C, taps]");
   auto sh = delta_shape(heads, kv_heads, dim, vdim, conv_w.size(1));
@@ -182,7 +182,7 @@ void delta_prep(Tensor qkv32, Tensor bg, Tensor x, Tensor b, Tensor a, Tensor co
   auto r = ragged(T, positions, cu_q, state_slots);
   HIP_OK(die::launch_delta_prep(qkv32.data_ptr<float>(), bg.data_ptr<float>(), x.data_ptr(), b.data_ptr(),
                                 a.data_ptr(), x.stride(0), f, f32_ptr(conv_w, C * sh.taps, "conv_w"),
-                                conv_state.data_ptr<float>(), f32_ptr(A_log, heads, "A_log"),
+                                f32_ptr(conv_wt, C * sh.taps, "conv_wt"), conv_state.data_ptr<float>(), f32_ptr(A_log, heads, "A_log"),
                                 f32_ptr(dt_bias, heads, "dt_bias"), sh, r, cur_stream()));
 }
 

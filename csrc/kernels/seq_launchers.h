@@ -66,10 +66,11 @@ struct DeltaShape {
 // before the step taken from conv_state [slots, taps - 1, C] (fp32, the most recent last); q and k heads made
 // unit vectors (q also times dim^-1/2); beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)).
 // Writes qkv32 [T, C] and bg [T, 2 * heads] = [beta | g], both fp32. A step with one row per sequence
-// (cu_q == nullptr) also moves the row's input into conv_state.
+// (cu_q == nullptr) also moves the row's input into conv_state. conv_w is [C, taps]; conv_wt, optional, the same
+// weights tap-major ([taps, C]), which lets prompt-sized bf16 steps load them 16 bytes at a time.
 hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void* b, const void* a, int64_t xstride,
-                             bool f32, const float* conv_w, float* conv_state, const float* A_log,
-                             const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s);
+                             bool f32, const float* conv_w, const float* conv_wt, float* conv_state,
+                             const float* A_log, const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s);
 // conv_state[slot(s)] = the last taps - 1 inputs of sequence s after this step (nothing to do when cu_q == nullptr)
 hipError_t launch_conv_state_update(float* conv_state, const void* x, int64_t xstride, bool f32, DeltaShape sh,
                                     RaggedRows r, hipStream_t s);

@@ -313,9 +313,9 @@ __global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void
 // ------------------------------------------------------------------------------------------ gated delta rule
 __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg, const void* x, const void* b,
                                                        const void* a, int64_t xstride, bool f32, const float* conv_w,
-                                                       float* conv_state, const float* A_log,
+                                                       const float* conv_wt, float* conv_state, const float* A_log,
                                                        const float* dt_bias, DeltaShape sh, RaggedRows r) {
-  extern __shared__ float vals[];  // [C]
+  extern __shared__ __attribute__((aligned(16))) float vals[];  // [C]
   const int row = blockIdx.x;
   const int s = seq_of_row(r.cu_q, r.num_seqs, row);
   const int first = r.cu_q ? r.cu_q[s] : s;
@@ -323,7 +323,32 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
   const int64_t p = r.positions[row];
   const int C = sh.channels(), taps = sh.taps;
   float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += NT) {
+  // prompt-sized bf16 steps with the weights also given tap-major ([taps, C]): 8 channels per thread and trip,
+  // 16-byte loads of inputs and weights
+  const bool wide = conv_wt != nullptr && r.cu_q != nullptr && !f32 && C % 8 == 0 && xstride % 8 == 0 && aligned16(x);
+  for (int c8 = threadIdx.x; wide && c8 < C / 8; c8 += NT) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      if (p - back < 0) continue;
+      const int src = i - back;
+      float xv[8];
+      if (src >= 0) {
+        unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + (int64_t)(row - back) * xstride + 8 * c8), xv);
+      } else {
+        const float4* sp = reinterpret_cast<const float4*>(st + (int64_t)(taps - 1 + src) * C + 8 * c8);
+        const float4 s0 = sp[0], s1 = sp[1];
+        xv[0] = s0.x, xv[1] = s0.y, xv[2] = s0.z, xv[3] = s0.w, xv[4] = s1.x, xv[5] = s1.y, xv[6] = s1.z, xv[7] = s1.w;
+      }
+      const float4* wp = reinterpret_cast<const float4*>(conv_wt + (int64_t)j * C + 8 * c8);
+      const float4 w0 = wp[0], w1 = wp[1];
+      acc[0] += w0.x * xv[0], acc[1] += w0.y * xv[1], acc[2] += w0.z * xv[2], acc[3] += w0.w * xv[3];
+      acc[4] += w1.x * xv[4], acc[5] += w1.y * xv[5], acc[6] += w1.z * xv[6], acc[7] += w1.w * xv[7];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) vals[8 * c8 + e] = rnd(siluf(rnd(acc[e], false)), false);
+  }
+  for (int c = threadIdx.x; !wide && c < C; c += NT) {
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int back = taps - 1 - j;
@@ -353,7 +378,12 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
     for (int c = lane; c < d; c += 64) v[c] *= sc;
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < C; c += NT) qkv32[(int64_t)row * C + c] = vals[c];
+  if (C % 4 == 0) {
+    float4* dst = reinterpret_cast<float4*>(qkv32 + (int64_t)row * C);
+    for (int c4 = threadIdx.x; c4 < C / 4; c4 += NT) dst[c4] = reinterpret_cast<const float4*>(vals)[c4];
+  } else {
+    for (int c = threadIdx.x; c < C; c += NT) qkv32[(int64_t)row * C + c] = vals[c];
+  }
   const int H = sh.heads;
   for (int h = threadIdx.x; h < H; h += NT) {
     const float bv = ldv(b, (int64_t)row * xstride + h, f32);
@@ -627,8 +657,8 @@ static bool delta_ok(const DeltaShape& sh) {
 }
 
 hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void* b, const void* a, int64_t xstride,
-                             bool f32, const float* conv_w, float* conv_state, const float* A_log,
-                             const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s) {
+                             bool f32, const float* conv_w, const float* conv_wt, float* conv_state,
+                             const float* A_log, const float* dt_bias, DeltaShape sh, RaggedRows r, hipStream_t s) {
   if (r.total_rows == 0) return hipSuccess;
   if (!delta_ok(sh) || !rows_ok(r)) return hipErrorInvalidValue;
   const size_t lds = sizeof(float) * sh.channels();
@@ -639,7 +669,7 @@ hipError_t launch_delta_prep(float* qkv32, float* bg, const void* x, const void*
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(delta_prep_kernel, dim3(r.total_rows), dim3(NT), lds, s, qkv32, bg, x, b, a, xstride, f32, conv_w,
-                     conv_state, A_log, dt_bias, sh, r);
+                     conv_wt, conv_state, A_log, dt_bias, sh, r);
   return hipGetLastError();
 }
 

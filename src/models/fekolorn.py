@@ -364,9 +364,12 @@ class GatedDeltaMixer:
         self.dt_bias = rnd(H, scale=0.5, dt=f32)
         self.norm = 1.0 + rnd(s.vdim, scale=0.1, dt=f32)
         self.o = rnd(hidden, H * s.vdim)
+        self.conv_wt = None
+        self.finalize()
 
     def finalize(self) -> None:
-        pass
+        """Derived tensors, after the weights changed: the convolution weights tap-major for 16-byte loads."""
+        self.conv_wt = self.conv_w.t().contiguous()
 
     def tensors(self) -> List[torch.Tensor]:
         return [self.w_in, self.conv_w, self.A_log, self.dt_bias, self.norm, self.o]
@@ -406,7 +409,7 @@ class GatedDeltaMixer:
         C, H = s.channels, s.heads
         x, b, a, g = p[:, :C], p[:, C: C + H], p[:, C + H: C + 2 * H], p[:, C + 2 * H: C + 2 * H + H * s.vdim]
         qkv32, bg = seq.delta_prep(x, b, a, self.conv_w, state["conv"], self.A_log, self.dt_bias, H, s.kv_heads, s.dim,
-                                   s.vdim, rag)
+                                   s.vdim, rag, conv_wt=self.conv_wt)
         seq.conv_state_update(state["conv"], x, H, s.kv_heads, s.dim, s.vdim, rag)
         o = seq.gated_delta(qkv32, bg, g, self.norm, eps, state["delta"], H, s.kv_heads, s.dim, s.vdim, rag)
         return mix.linear(o, self.o)

@@ -149,18 +149,19 @@ def poly_norm_act(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tens
 # ---------------------------------------------------------------------------------------------- gated delta rule
 def delta_prep(x: torch.Tensor, b: torch.Tensor, a: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Tensor,
                A_log: torch.Tensor, dt_bias: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int,
-               rag: Ragged) -> Tuple[torch.Tensor, torch.Tensor]:
+               rag: Ragged, conv_wt: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """x [T, C = 2 G dim + H vdim] = [q | k | v] channels: causal convolution over the sequence's last ``taps``
     inputs (those before the step from conv_state [slots, taps - 1, C]) + SiLU; q and k heads to unit length
     (q also times dim^-1/2). Returns (qkv32 [T, C] fp32, bg [T, 2 H] fp32 = [sigmoid(b) | exp(-exp(A_log) *
     softplus(a + dt_bias))]). On the GPU a step with one row per sequence also moves the row's input into
-    conv_state (:func:`conv_state_update` then has nothing left to do)."""
+    conv_state (:func:`conv_state_update` then has nothing left to do). ``conv_wt``: the same weights tap-major,
+    [taps, C] contiguous, which lets the kernel load them 16 bytes at a time in prompt-sized bf16 steps."""
     T, C = x.shape
     taps = conv_w.shape[1]
     qkv32 = torch.empty(T, C, dtype=torch.float32, device=x.device)
     bg = torch.empty(T, 2 * heads, dtype=torch.float32, device=x.device)
     if x.is_cuda:
-        _kern().delta_prep(qkv32, bg, x, b, a, conv_w, conv_state, A_log, dt_bias, heads, kv_heads, dim, vdim,
+        _kern().delta_prep(qkv32, bg, x, b, a, conv_w, conv_wt, conv_state, A_log, dt_bias, heads, kv_heads, dim, vdim,
                            rag.positions, rag.cu_q, rag.state_slots)
         return qkv32, bg
     pos = rag.positions.tolist()

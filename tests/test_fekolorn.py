@@ -308,6 +308,15 @@ def test_gated_delta_rule_in_portions_and_slots(device, shape):
                          torch.tensor(slots, dtype=torch.int32, device=device))
         x, b, a, gt = p[:, :C], p[:, C: C + H], p[:, C + H: C + 2 * H], p[:, C + 2 * H:]
         qkv32, bg = seq.delta_prep(x, b, a, conv_w, state["conv"], f(w["A_log"]), f(w["dt_bias"]), H, G, d, dv, rag)
+        if not single:   # the tap-major weights (16-byte path of bf16 prompt steps) give the same as the plain ones
+            xb, bb, ab = x.bfloat16(), b.bfloat16(), a.bfloat16()
+            pad = xb.new_zeros(xb.shape[0], (-(C + 2 * H)) % 8)   # a row stride that allows 16-byte loads
+            pb = torch.cat([xb, bb, ab, pad], 1)
+            xb, bb, ab = pb[:, :C], pb[:, C: C + H], pb[:, C + H: C + 2 * H]
+            ref32, _ = seq.delta_prep(xb, bb, ab, conv_w, state["conv"], f(w["A_log"]), f(w["dt_bias"]), H, G, d, dv, rag)
+            got32, _ = seq.delta_prep(xb, bb, ab, conv_w, state["conv"], f(w["A_log"]), f(w["dt_bias"]), H, G, d, dv, rag,
+                                      conv_wt=conv_w.t().contiguous())
+            assert torch.allclose(ref32, got32, atol=1e-6), float((ref32 - got32).abs().max())
         seq.conv_state_update(state["conv"], x, H, G, d, dv, rag)
         o = seq.gated_delta(qkv32, bg, gt, f(w["norm"]), eps, state["delta"], H, G, d, dv, rag).cpu().double()
         r = 0
