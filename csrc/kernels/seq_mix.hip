@@ -311,6 +311,8 @@ __global__ void __launch_bounds__(NT) poly_norm_act_kernel(void* out, const void
 }
 
 // ------------------------------------------------------------------------------------------ gated delta rule
+constexpr int TAPS_MAX = 16;
+
 __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg, const void* x, const void* b,
                                                        const void* a, int64_t xstride, bool f32, const float* conv_w,
                                                        const float* conv_wt, float* conv_state, const float* A_log,
@@ -323,9 +325,9 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
   const int64_t p = r.positions[row];
   const int C = sh.channels(), taps = sh.taps;
   float* st = conv_state + (int64_t)r.state_slots[s] * (taps - 1) * C;
-  // prompt-sized bf16 steps with the weights also given tap-major ([taps, C]): 8 channels per thread and trip,
-  // 16-byte loads of inputs and weights
-  const bool wide = conv_wt != nullptr && r.cu_q != nullptr && !f32 && C % 8 == 0 && xstride % 8 == 0 && aligned16(x);
+  // bf16 steps with the weights also given tap-major ([taps, C]): 8 channels per thread and trip, 16-byte loads of
+  // inputs, weights and state (a decode row is then two dependent trips per thread instead of C / 256)
+  const bool wide = conv_wt != nullptr && !f32 && C % 8 == 0 && xstride % 8 == 0 && aligned16(x);
   for (int c8 = threadIdx.x; wide && c8 < C / 8; c8 += NT) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < taps; ++j) {
@@ -340,6 +342,7 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
         const float4 s0 = sp[0], s1 = sp[1];
         xv[0] = s0.x, xv[1] = s0.y, xv[2] = s0.z, xv[3] = s0.w, xv[4] = s1.x, xv[5] = s1.y, xv[6] = s1.z, xv[7] = s1.w;
       }
+
       const float4* wp = reinterpret_cast<const float4*>(conv_wt + (int64_t)j * C + 8 * c8);
       const float4 w0 = wp[0], w1 = wp[1];
       acc[0] += w0.x * xv[0], acc[1] += w0.y * xv[1], acc[2] += w0.z * xv[2], acc[3] += w0.w * xv[3];
@@ -347,6 +350,26 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) vals[8 * c8 + e] = rnd(siluf(rnd(acc[e], false)), false);
+    if (r.cu_q == nullptr) {
+      // one row per sequence: this thread is the only reader of its channels' tail, so it shifts it here: state
+      // row k takes row k + 1 (zeros where that lies before the sequence's start), the last one the row's input
+      const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int k = 0; k + 1 < taps - 1; ++k) {
+        const bool live = p - (taps - 2 - k) >= 0;
+        float4* dp = reinterpret_cast<float4*>(st + (int64_t)k * C + 8 * c8);
+        const float4* sp = reinterpret_cast<const float4*>(st + (int64_t)(k + 1) * C + 8 * c8);
+        const float4 t0 = sp[0], t1 = sp[1];
+        dp[0] = live ? t0 : zero;
+        dp[1] = live ? t1 : zero;
+      }
+      if (taps > 1) {
+        float xv[8];
+        unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + (int64_t)row * xstride + 8 * c8), xv);
+        float4* dp = reinterpret_cast<float4*>(st + (int64_t)(taps - 2) * C + 8 * c8);
+        dp[0] = make_float4(xv[0], xv[1], xv[2], xv[3]);
+        dp[1] = make_float4(xv[4], xv[5], xv[6], xv[7]);
+      }
+    }
   }
   for (int c = threadIdx.x; !wide && c < C; c += NT) {
     float acc = 0.f;
@@ -393,8 +416,6 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(float* qkv32, float* bg,
     bg[(int64_t)row * 2 * H + H + h] = expf(-expf(A_log[h]) * sp);
   }
 }
-
-constexpr int TAPS_MAX = 16;
 
 __global__ void __launch_bounds__(NT) conv_state_update_kernel(float* conv_state, const void* x, int64_t xstride,
                                                               bool f32, DeltaShape sh, RaggedRows r) {
