@@ -574,25 +574,58 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
   const int64_t t = blockIdx.x;
   const bool f32 = a.f32;
   float sq = 0.f, sk = 0.f;
-  for (int c = threadIdx.x; c < nq; c += NT) {
-    const float x = ldv(a.q, t * a.xstride + c, f32);
-    qv[c] = x;
-    sq += x * x;
-  }
-  for (int c = threadIdx.x; c < nk; c += NT) {
-    const float x = ldv(a.k, t * a.xstride + c, f32);
-    kv[c] = x;
-    sk += x * x;
-  }
   float lam = 0.f;
   if (a.v_lambda != nullptr) lam = a.v_lambda[0];
-  for (int c = threadIdx.x; c < nv; c += NT) {
-    float x = ldv(a.v, t * a.xstride + c, f32);
-    if (a.v_lambda != nullptr) x = (1.0f - lam) * x + lam * ldv(a.v_first, t * a.vfstride + c, f32);
-    vv[c] = x;
+  // bf16 with head sizes that are multiples of 8: 16-byte loads and stores, 8 values per thread and trip
+  const bool wide = !f32 && d % 8 == 0 && dv % 8 == 0 && a.xstride % 8 == 0 && aligned16(a.q) && aligned16(a.k) &&
+                    aligned16(a.v) && aligned16(a.q_out) && aligned16(a.cache) &&
+                    (a.v_first == nullptr || (a.vfstride % 8 == 0 && aligned16(a.v_first)));
+  if (wide) {
+    const bf16_t* qp = reinterpret_cast<const bf16_t*>(a.q) + t * a.xstride;
+    const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.k) + t * a.xstride;
+    const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.v) + t * a.xstride;
+    for (int c8 = threadIdx.x; c8 < (nq + nk + nv) / 8; c8 += NT) {
+      const int c = 8 * c8;
+      float f[8];
+      if (c < nq) {
+        unpack8(*reinterpret_cast<const uint4*>(qp + c), f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += f[e] * f[e];
+      } else if (c < nq + nk) {
+        unpack8(*reinterpret_cast<const uint4*>(kp + c - nq), f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sk += f[e] * f[e];
+      } else {
+        unpack8(*reinterpret_cast<const uint4*>(vp + c - nq - nk), f);
+        if (a.v_lambda != nullptr) {
+          float g8[8];
+          unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(a.v_first) + t * a.vfstride + c - nq - nk), g8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) f[e] = (1.0f - lam) * f[e] + lam * g8[e];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[c + e] = f[e];   // qv, kv and vv are adjacent
+    }
+  } else {
+    for (int c = threadIdx.x; c < nq; c += NT) {
+      const float x = ldv(a.q, t * a.xstride + c, f32);
+      qv[c] = x;
+      sq += x * x;
+    }
+    for (int c = threadIdx.x; c < nk; c += NT) {
+      const float x = ldv(a.k, t * a.xstride + c, f32);
+      kv[c] = x;
+      sk += x * x;
+    }
+    for (int c = threadIdx.x; c < nv; c += NT) {
+      float x = ldv(a.v, t * a.xstride + c, f32);
+      if (a.v_lambda != nullptr) x = (1.0f - lam) * x + lam * ldv(a.v_first, t * a.vfstride + c, f32);
+      vv[c] = x;
+    }
   }
   if (a.q_norm != nullptr) {
-    sq = block_sum<NT>(sq, red);
+    sq = block_sum<NT>(sq, red);   // (a barrier: every thread's loads are in LDS)
     sk = block_sum<NT>(sk, red);
     const float rq = 1.0f / sqrtf(sq / (float)nq + a.eps), rk = 1.0f / sqrtf(sk / (float)nk + a.eps);
     for (int c = threadIdx.x; c < nq; c += NT) qv[c] *= rq * a.q_norm[c];
@@ -623,11 +656,24 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < nq; c += NT) stv(a.q_out, t * nq + c, f32, qv[c]);
   const int64_t slot = a.slots[t];
-  if (slot < 0) return;
   // the block's interior is head-major: [G][block_size][K | V]
   const int64_t blk = slot / a.block_size, off = slot % a.block_size;
+  if (wide) {
+    bf16_t* qo = reinterpret_cast<bf16_t*>(a.q_out) + t * nq;
+    for (int c8 = threadIdx.x; c8 < nq / 8; c8 += NT) *reinterpret_cast<uint4*>(qo + 8 * c8) = pack8(qv + 8 * c8);
+    if (slot < 0) return;
+    bf16_t* cb = reinterpret_cast<bf16_t*>(a.cache);
+    for (int c8 = threadIdx.x; c8 < (nk + nv) / 8; c8 += NT) {
+      const int c = 8 * c8;
+      const int g = c < nk ? c / d : (c - nk) / dv;
+      const int e = c < nk ? c % d : d + (c - nk) % dv;
+      *reinterpret_cast<uint4*>(cb + ((blk * G + g) * a.block_size + off) * (int64_t)(d + dv) + e) = pack8(kv + c);
+    }
+    return;
+  }
+  for (int c = threadIdx.x; c < nq; c += NT) stv(a.q_out, t * nq + c, f32, qv[c]);
+  if (slot < 0) return;
   for (int c = threadIdx.x; c < nk + nv; c += NT) {
     const int g = c < nk ? c / d : (c - nk) / dv;
     const int e = c < nk ? c % d : d + (c - nk) % dv;
