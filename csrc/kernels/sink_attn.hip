@@ -323,6 +323,9 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   const char* vbase = reinterpret_cast<const char*>(ks) + (4 * hh + (i16 >> 2)) * pitchB +
                       (D + 16 * (g16 & 1) + 4 * (i16 & 3)) * 2;
   const float* bias = a.bias ? a.bias + myh : nullptr;
+  // distances from bias_rows - 1 on share the table's last row: a lane whose 16 keys of a tile all lie that far
+  // back adds that one value without looking anything up
+  const float bias_far = bias ? bias[(int64_t)(a.bias_rows - 1) * H] * LOG2E : 0.f;
   // a tile is interior for a wave when every one of its 32 x 32 (key, row) pairs is visible: no masking then
   const int wrow_first = row0 + wave * 32, wrow_last = wrow_first + 31;
   const bool wave_full = wrow_last < nrows;
@@ -360,15 +363,22 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
     const bool interior = wave_full && j0 + MKT - 1 <= min(pw_first, jhi) &&
                           (a.window <= 0 || pw_last - j0 < a.window);
     if (interior) {
+      const bool far = bias == nullptr || prow - (j0 + 27 + 4 * hh) >= a.bias_rows - 1;
+      if (far) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = sc[r] * sl2;
-        if (bias != nullptr) {
-          const int n = prow - (j0 + (r & 3) + 8 * (r >> 2) + 4 * hh);
-          v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+        for (int r = 0; r < 16; ++r) {
+          const float v = sc[r] * sl2 + bias_far;
+          sc[r] = v;
+          mx = fmaxf(mx, v);
         }
-        sc[r] = v;
-        mx = fmaxf(mx, v);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = prow - (j0 + (r & 3) + 8 * (r >> 2) + 4 * hh);
+          const float v = sc[r] * sl2 + bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+          sc[r] = v;
+          mx = fmaxf(mx, v);
+        }
       }
     } else {
 #pragma unroll

@@ -336,7 +336,7 @@ def _paged(device, dtype, n_blocks, bs, width, seed):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", ["rotary", "biased", "wide", "mc_rotary", "mc_biased", "served_rotary", "served_biased"])
+@pytest.mark.parametrize("case", ["rotary", "biased", "wide", "mc_rotary", "mc_biased", "served_rotary", "served_biased", "mc_far_bias"])
 def test_attention_ops_with_standout_keys(device, dtype, case):
     """qkv_prep + sink_attn over scattered pages, prompt portion and single decode rows: one key far back, one on a
     page border, and the keys just inside and just outside the window are made to stand out (their scores lead by
@@ -353,6 +353,8 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
         H, G, d, dv, window, rot, bias_max = 8, 2, 80, 32, 0, 48, 0
     elif case == "mc_biased":
         H, G, d, dv, window, rot, bias_max = 6, 2, 32, 96, 37, 0, 15.0
+    elif case == "mc_far_bias":    # a window several times the bias table's reach: whole tiles share its last row
+        H, G, d, dv, window, rot, bias_max = 4, 2, 32, 32, 80, 0, 6.0
     elif case == "served_rotary":  # default dispatch at a served shape: 8 query heads on one key/value head
         H, G, d, dv, window, rot, bias_max = 8, 1, 128, 128, 0, 64, 0
     elif case == "served_biased":  # default dispatch, one query head per key/value head
@@ -360,7 +362,7 @@ def test_attention_ops_with_standout_keys(device, dtype, case):
     else:
         H, G, d, dv, window, rot, bias_max = 2, 1, 96, 160, 40, 0, 0
     impl = 2 if case.startswith("mc_") and dtype == torch.bfloat16 and device != "cpu" else 0
-    rotary, biased = case.endswith("rotary"), case.endswith("biased")
+    rotary, biased = case.endswith("rotary"), case.endswith("biased") or case.endswith("bias")
     T, bs = 90, 8
     g = torch.Generator().manual_seed(len(case))
     q = torch.randn(T, H, d, generator=g) * 0.3
